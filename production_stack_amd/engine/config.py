@@ -42,6 +42,21 @@ class MixerSpec:
     (general_delta), `conv` the taps of the short causal convolution on
     q/k/v and `gate_rank` the width of the low-rank output gate
     (channel_delta).
+    Attention with `rope` and `rot_dims` > 0 turns the first `rot_dims`
+    entries of every query and key head (interleaved pairs, base
+    `rot_base`, positions divided by `rot_factor`); `out_gate` multiplies
+    the concatenated heads by sigmoid(W_g h), `out_bias` adds a bias to the
+    output projection.
+    kind "gla" / "ssd" / "mlstm": gated linear recurrences without a
+    removal term (state heads x dim x vdim): "gla" decays every key channel
+    by sigmoid(low-rank projection of width `decay_rank`)^(1/`tau`); "ssd"
+    is the state-space-duality mixer (`state` = dim entries per head,
+    keys/queries shared by `groups` groups, convolution of `conv` taps, one
+    step size and decay per head, gated read-out normalised in
+    `norm_groups` parts); "mlstm" has exponential input/forget gates capped
+    at +-`gate_cap`, a running maximum and a normaliser.
+    kind "pair": two mixers `left` and `right` read the same input; the
+    result is the mean of their separately normalised outputs.
     """
 
     kind: str
@@ -68,6 +83,16 @@ class MixerSpec:
     rot_base: float = 10000.0
     conv: int = 0
     gate_rank: int = 0
+    rot_factor: float = 1.0
+    out_gate: bool = False
+    out_bias: bool = False
+    state: int = 0
+    groups: int = 0
+    norm_groups: int = 1
+    tau: float = 1.0
+    gate_cap: float = 0.0
+    left: Optional["MixerSpec"] = None
+    right: Optional["MixerSpec"] = None
 
 
 @dataclass
@@ -77,7 +102,11 @@ class MlpSpec:
     routed by `score` ("softmax" | "sigmoid") with optional renormalised
     weights applied to the expert's output or (`weight_on_input`) input;
     an always-on shared expert of width `shared_ff` may be added, scaled by
-    a per-token sigmoid gate."""
+    a per-token sigmoid gate. `correction`: a learned per-expert offset
+    joins the scores for the choice only; `identity`: that many extra
+    router outputs (after the experts) stand for experts that return their
+    input; `route_scale` multiplies the final weights; `renorm_eps` is
+    added to the sum the chosen weights are divided by."""
 
     kind: str
     ff: int
@@ -90,6 +119,10 @@ class MlpSpec:
     weight_on_input: bool = False
     shared_ff: int = 0
     shared_limit: float = 0.0
+    correction: bool = False
+    identity: int = 0
+    route_scale: float = 1.0
+    renorm_eps: float = 0.0
 
 
 @dataclass
@@ -105,6 +138,10 @@ class LayerSpec:
     # the layer hands on a learned weighted sum of the embedding output and
     # all layer results so far instead of its own result
     depth_average: bool = False
+    # every sublayer's output is RMS-normalised (own weight) before it
+    # joins the residual stream, and then scaled per channel (`layer_scale`)
+    post_norm: bool = False
+    layer_scale: bool = False
 
 
 @dataclass
@@ -143,6 +180,8 @@ class ModelConfig:
     # RMS norms of the stack normalise this many equal consecutive parts
     # of the vector separately
     norm_groups: int = 1
+    # logits become cap * tanh(logits / cap) (0 = off)
+    logit_softcap: float = 0.0
 
     @property
     def has_recurrent_state(self) -> bool:

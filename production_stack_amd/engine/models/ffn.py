@@ -26,13 +26,23 @@ from production_stack_amd.ops import gemm_policy
 
 
 def route(x: torch.Tensor, router_w: torch.Tensor, top: int,
-          score: str = "softmax", renormalize: bool = True):
+          score: str = "softmax", renormalize: bool = True,
+          correction: Optional[torch.Tensor] = None, scale: float = 1.0,
+          renorm_eps: float = 0.0):
     """Returns (weights fp32 [T, top], expert ids [T, top]). The logits are
-    an fp32 product of the (up-cast) activations and router weights."""
+    an fp32 product of the (up-cast) activations and router weights.
+    correction (fp32 [experts]): added to the softmax scores for the choice
+    only, the weights are the plain scores; the chosen weights are divided
+    by (their sum + renorm_eps) when renormalize, then multiplied by
+    scale."""
     logits = F.linear(x.float(), router_w.float())
     if score == "softmax":
         probs = torch.softmax(logits, dim=-1)
-        weights, sel = torch.topk(probs, top, dim=-1)
+        if correction is not None:
+            _, sel = torch.topk(probs + correction, top, dim=-1)
+            weights = probs.gather(-1, sel)
+        else:
+            weights, sel = torch.topk(probs, top, dim=-1)
     elif score == "sigmoid":
         # rank by the logits: the sigmoid is monotonic but saturates to
         # exactly 1.0 in fp32, which would tie large scores
@@ -41,7 +51,9 @@ def route(x: torch.Tensor, router_w: torch.Tensor, top: int,
     else:
         raise ValueError(f"unknown router score {score!r}")
     if renormalize:
-        weights = weights / weights.sum(dim=-1, keepdim=True)
+        weights = weights / (weights.sum(dim=-1, keepdim=True) + renorm_eps)
+    if scale != 1.0:
+        weights = weights * scale
     return weights, sel
 
 
@@ -74,6 +86,9 @@ def sparse_moe(x: torch.Tensor, weights: torch.Tensor, sel: torch.Tensor,
         if weight_on_input:
             xe = (xe.float() * w.unsqueeze(-1)).to(x.dtype)
             ye = expert_fn(e, xe)
+        elif out.dtype == torch.float32:
+            # fp32 accumulator: the fp32 routing weight is applied unrounded
+            ye = expert_fn(e, xe).float() * w.unsqueeze(-1)
         else:
             ye = expert_fn(e, xe) * w.to(x.dtype).unsqueeze(-1)
         out.index_add_(0, rows, ye.to(out.dtype))
@@ -110,13 +125,19 @@ class GatedMLP(nn.Module):
 
 class SparseMoE(nn.Module):
     """Routed experts (+ optional always-on shared expert scaled by a
-    per-token sigmoid gate), configured by an MlpSpec."""
+    per-token sigmoid gate), configured by an MlpSpec. The router may have
+    `identity` outputs beyond the experts: choosing one of them returns
+    the (weighted) input itself."""
 
     def __init__(self, width: int, spec: MlpSpec, dtype: torch.dtype) -> None:
         super().__init__()
         self.spec = spec
         E, ff = spec.experts, spec.ff
-        self.router = nn.Parameter(torch.empty(E, width, dtype=dtype))
+        self.router = nn.Parameter(
+            torch.empty(E + spec.identity, width, dtype=dtype))
+        self.correction = (
+            nn.Parameter(torch.empty(E + spec.identity, dtype=torch.float32))
+            if spec.correction else None)
         self.experts_gate_up = nn.Parameter(
             torch.empty(E, 2 * ff, width, dtype=dtype))
         self.experts_down = nn.Parameter(
@@ -127,6 +148,26 @@ class SparseMoE(nn.Module):
                                    spec.shared_limit, dtype)
             self.shared_gate = nn.Parameter(
                 torch.empty(1, width, dtype=dtype))
+        self._fused_in = None
+
+    def _apply(self, fn, *a, **kw):
+        # the fused input weight is a plain tensor rebuilt after a move
+        self._fused_in = None
+        return super()._apply(fn, *a, **kw)
+
+    def fused_in(self) -> torch.Tensor:
+        """The shared expert's gate | up | scalar-gate rows as one weight;
+        the parts become views of it."""
+        w = self._fused_in
+        if w is None:
+            parts = self.in_params()
+            w = torch.cat([p.data for p in parts], dim=0).contiguous()
+            off = 0
+            for p in parts:
+                p.data = w[off:off + p.shape[0]]
+                off += p.shape[0]
+            self._fused_in = w
+        return w
 
     def in_params(self):
         """Parameters the caller may fold into a fused projection of the
@@ -149,9 +190,11 @@ class SparseMoE(nn.Module):
         biases: a zero-weighted input (or output) contributes exactly 0."""
         sp = self.spec
         T, E, ff = x.shape[0], sp.experts, sp.ff
-        wm = torch.zeros((T, E), dtype=torch.float32, device=x.device)
+        wm = torch.zeros((T, E + sp.identity), dtype=torch.float32,
+                         device=x.device)
         wm.scatter_(1, sel, weights)
-        wm = wm.t().unsqueeze(-1)                       # [E, T, 1]
+        w_id = wm[:, E:].sum(dim=1, keepdim=True) if sp.identity else None
+        wm = wm[:, :E].t().unsqueeze(-1)                # [E, T, 1]
         if sp.weight_on_input:
             xe = (x.float().unsqueeze(0) * wm).to(x.dtype)
         else:
@@ -163,9 +206,14 @@ class SparseMoE(nn.Module):
         y = y.float()
         if not sp.weight_on_input:
             y = y * wm
-        return y.sum(dim=0)
+        y = y.sum(dim=0)
+        if w_id is not None:
+            y += x.float() * w_id
+        return y
 
     def _expert(self, e: int, xe: torch.Tensor) -> torch.Tensor:
+        if e >= self.spec.experts:      # identity expert
+            return xe
         ff = self.spec.ff
         gu = gemm_policy.linear(xe, self.experts_gate_up[e])
         act = ops.gated_act(gu[:, :ff], gu[:, ff:], self.spec.act,
@@ -180,13 +228,15 @@ class SparseMoE(nn.Module):
         fp32."""
         sp = self.spec
         weights, sel = route(x, self.router, sp.top, sp.score,
-                             sp.renormalize)
+                             sp.renormalize, self.correction,
+                             sp.route_scale, sp.renorm_eps)
         T = x.shape[0]
         if T <= self.DENSE_MAX_ROWS and T * sp.top >= sp.experts:
             out = self._all_experts(x, weights, sel)
         else:
             out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
-            sparse_moe(x, weights, sel, sp.experts, self._expert,
+            sparse_moe(x, weights, sel, sp.experts + sp.identity,
+                       self._expert,
                        weight_on_input=sp.weight_on_input, out=out)
         if self.shared is not None:
             sff = sp.shared_ff
@@ -196,7 +246,6 @@ class SparseMoE(nn.Module):
         return out
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        ps = self.in_params()
-        proj = (gemm_policy.linear(x, torch.cat(list(ps), dim=0))
-                if ps else None)
+        proj = (gemm_policy.linear(x, self.fused_in())
+                if self.shared is not None else None)
         return self.forward_from_proj(x, proj)

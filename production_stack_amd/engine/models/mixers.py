@@ -35,31 +35,42 @@ DELTA_DECAY_SCALE = math.exp(-0.5)
 
 class TalkAttention(nn.Module):
     """Grouped-query softmax attention over the paged KV cache with the
-    MixerSpec's options: no rotary code, score mixing across heads,
-    aligned-chunk / trailing-window visibility (with kept first keys),
-    capped scores, denominator sink (fixed or learned), projection biases,
-    per-head query/key norm, value blending with the stack's first
-    value-mixing layer; key and value widths may differ."""
+    MixerSpec's options: score mixing across heads, aligned-chunk /
+    trailing-window visibility (with kept first keys), capped scores,
+    denominator sink (fixed or learned), projection biases, per-head
+    query/key norm, rotary position code on the leading entries of every
+    head (interleaved pairs, linear position scaling), value blending with
+    the stack's first value-mixing layer, a sigmoid output gate on the
+    concatenated heads; key and value widths may differ."""
 
     kind = "attention"
 
     def __init__(self, width: int, spec: MixerSpec,
-                 dtype: torch.dtype, eps: float = 1e-5) -> None:
+                 dtype: torch.dtype, eps: float = 1e-5,
+                 max_pos: int = 8192) -> None:
         super().__init__()
-        if spec.rope:
+        if spec.rope and spec.rot_dims <= 0:
             raise NotImplementedError(
-                "TalkAttention carries no rotary code; rope layers use the "
+                "rotary attention here turns interleaved pairs of the "
+                "first rot_dims entries; the half-split layout is the "
                 "Llama attention path")
         self.spec = spec
+        self.max_pos = max_pos
+        self._cos_sin = None
         H, G = spec.heads, spec.kv_heads or spec.heads
         D, DV = spec.dim, spec.vdim or spec.dim
         if H % G:
             raise ValueError("heads must be a multiple of kv_heads")
         self.H, self.G, self.D, self.DV = H, G, D, DV
-        self.qkv = nn.Parameter(
-            torch.empty(H * D + G * D + G * DV, width, dtype=dtype))
+        # fused rows: q | k | v (| output gate)
+        self.qkv_rows = H * D + G * D + G * DV
+        self.qkv = nn.Parameter(torch.empty(
+            self.qkv_rows + (H * DV if spec.out_gate else 0), width,
+            dtype=dtype))
         self.out_weight = nn.Parameter(
             torch.empty(width, H * DV, dtype=dtype))
+        self.out_bias = (nn.Parameter(torch.empty(width, dtype=dtype))
+                         if spec.out_bias else None)
         self.talk = (
             nn.Parameter(torch.empty(H, H, dtype=torch.float32))
             if spec.talking_heads else None)
@@ -81,6 +92,25 @@ class TalkAttention(nn.Module):
 
     def in_params(self):
         return [self.qkv]
+
+    def in_bias(self):
+        return self.qkv_bias
+
+    def cos_sin(self, device) -> Optional[torch.Tensor]:
+        sp = self.spec
+        if not sp.rope:
+            return None
+        cs = self._cos_sin
+        if cs is None or cs.device != device:
+            cs = ops.rope_table(self.max_pos, sp.rot_dims, sp.rot_base,
+                                device, sp.rot_factor)
+            self._cos_sin = cs
+        return cs
+
+    def project(self, o: torch.Tensor) -> torch.Tensor:
+        if self.out_bias is not None:
+            return torch.addmm(self.out_bias, o, self.out_weight.t())
+        return gemm_policy.linear(o, self.out_weight)
 
     def forward(self, h: torch.Tensor, meta, cache, shared: dict,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -105,15 +135,18 @@ class TalkAttention(nn.Module):
         k_cache, v_cache = cache
         q = proj[:, :H * D]
         k = proj[:, H * D:H * D + G * D]
-        v = proj[:, H * D + G * D:]
+        v = proj[:, H * D + G * D:self.qkv_rows]
         sp = self.spec
-        if sp.qk_norm or sp.v_mix:
+        if sp.qk_norm or sp.v_mix or sp.rope:
             # the first value-mixing layer of a step publishes its values;
             # later ones blend theirs with them before caching
             v_first = shared.get("v_first") if sp.v_mix else None
             ops.attn_prep(q, k, v, self.q_norm, self.k_norm, self.eps,
                           self.vmix, v_first, k_cache, v_cache,
-                          meta.slot_mapping, H)
+                          meta.slot_mapping, H,
+                          cos_sin=self.cos_sin(proj.device),
+                          positions=meta.positions,
+                          rot_dims=sp.rot_dims if sp.rope else 0)
             if sp.v_mix and v_first is None:
                 shared["v_first"] = v
         else:
@@ -136,6 +169,8 @@ class TalkAttention(nn.Module):
                     talk=self.talk, out=out[a:b], variant=variant,
                     keep_first=sp.keep_first, softcap=sp.softcap,
                     sink_vals=self.sink_vals)
+        if sp.out_gate:
+            ops.gated_act(proj[:, self.qkv_rows:], out, "sigmoid", out=out)
         return out
 
 
@@ -346,10 +381,251 @@ class ChannelDelta(nn.Module):
             state, meta.seq_rows, H, G, self.eps, out=out)
 
 
+class _ScanMixer(nn.Module):
+    """Shared plumbing of the gated linear recurrences: one fused input
+    projection, a per-sequence fp32 state heads x dim x vdim, one output
+    projection."""
+
+    def in_params(self):
+        return [self.in_proj]
+
+    def in_bias(self):
+        return None
+
+    @property
+    def out_in(self) -> int:
+        return self.H * self.DV
+
+    def project(self, o: torch.Tensor) -> torch.Tensor:
+        return gemm_policy.linear(o, self.out_weight)
+
+    def forward(self, h: torch.Tensor, meta, cache, shared: dict,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return self.forward_from_proj(gemm_policy.linear(h, self.in_proj),
+                                      meta, cache, out)
+
+
+class GatedLinearAttention(_ScanMixer):
+    """Linear attention whose state rows decay per key channel:
+    alpha = sigmoid(W_a2 W_a1 h + b)^(1/tau), S <- diag(alpha) S + k v^T,
+    o = S^T (q dim^-1/2); o is RMS-normalised per head (weight shared by
+    the heads) and multiplied by silu(W_g h)."""
+
+    kind = "gla"
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float,
+                 dtype: torch.dtype) -> None:
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        H, D, DV = spec.heads, spec.dim, spec.vdim or spec.dim
+        self.H, self.D, self.DV, self.R = H, D, DV, spec.decay_rank
+        # fused rows: q | k | v | output gate | decay rank
+        self.in_proj = nn.Parameter(torch.empty(
+            2 * H * D + 2 * H * DV + self.R, width, dtype=dtype))
+        self.a2 = nn.Parameter(torch.empty(H * D, self.R, dtype=dtype))
+        self.a_bias = nn.Parameter(torch.empty(H * D, dtype=torch.float32))
+        self.out_norm = nn.Parameter(torch.empty(DV, dtype=torch.float32))
+        self.out_weight = nn.Parameter(
+            torch.empty(width, H * DV, dtype=dtype))
+
+    def cache_shape(self):
+        return ("state", self.H, self.D, self.DV)
+
+    def forward_from_proj(self, proj, meta, cache, out=None):
+        H, D, DV = self.H, self.D, self.DV
+        a, b, c = H * D, 2 * H * D, 2 * H * D + H * DV
+        z = gemm_policy.linear(proj[:, c + H * DV:], self.a2)
+        return ops.linear_scan(
+            "gla", proj[:, :a], proj[:, a:b], proj[:, b:c], z,
+            proj[:, c:c + H * DV], cache, meta.seq_rows, H, H, self.eps,
+            qscale=D ** -0.5, c0=1.0 / self.spec.tau, p0=self.a_bias,
+            normw=self.out_norm, out=out)
+
+
+class MatrixLSTM(_ScanMixer):
+    """Matrix-memory LSTM: per head log gates i = cap(W_i h + b_i),
+    f = logsigmoid(cap(W_f h + b_f)), cap(z) = c tanh(z / c); with the
+    running maximum m' = max(f + m, i) (m starts at 0) the memory and its
+    normaliser are S <- e^(f+m-m') S + e^(i-m') k v^T, n likewise with k;
+    o = S^T q / (max(|n.q|, e^-m') + 1e-6), q scaled by dim^-1/2; o is
+    divided by its per-head root mean square, scaled by a weight over all
+    heads and by sigmoid(W_g h). Per sequence: S plus (n, m)."""
+
+    kind = "mlstm"
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float,
+                 dtype: torch.dtype) -> None:
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        H, D, DV = spec.heads, spec.dim, spec.vdim or spec.dim
+        self.H, self.D, self.DV = H, D, DV
+        # fused rows: q | k | v | output gate | input gate | forget gate
+        self.in_proj = nn.Parameter(torch.empty(
+            2 * H * D + 2 * H * DV + 2 * H, width, dtype=dtype))
+        self.i_bias = nn.Parameter(torch.empty(H, dtype=torch.float32))
+        self.f_bias = nn.Parameter(torch.empty(H, dtype=torch.float32))
+        self.out_norm = nn.Parameter(torch.empty(H * DV,
+                                                 dtype=torch.float32))
+        self.out_weight = nn.Parameter(
+            torch.empty(width, H * DV, dtype=dtype))
+
+    def cache_shape(self):
+        return ("multi", [("state", self.H, self.D, self.DV),
+                          ("slots", (self.H, self.D + 1), torch.float32)])
+
+    def forward_from_proj(self, proj, meta, cache, out=None):
+        H, D, DV = self.H, self.D, self.DV
+        a, b, c = H * D, 2 * H * D, 2 * H * D + H * DV
+        e = c + H * DV
+        state, aux = cache
+        return ops.linear_scan(
+            "mlstm", proj[:, :a], proj[:, a:b], proj[:, b:c],
+            proj[:, e + H:e + 2 * H], proj[:, c:e], state, meta.seq_rows,
+            H, H, self.eps, qscale=D ** -0.5, c0=self.spec.gate_cap,
+            wr=proj[:, e:e + H], p0=self.i_bias, p1=self.f_bias,
+            normw=self.out_norm, aux=aux, out=out)
+
+
+class StateSpaceDuality(_ScanMixer):
+    """State-space-duality mixer (scalar decay per head): the input
+    projection gives z | x | B | C | dt; x, B, C pass a short causal
+    convolution (with bias) and silu; dt = softplus(dt + dt_bias);
+    S <- exp(-exp(A_log) dt) S + dt B x^T (state x vdim per head, B and C
+    shared by groups of heads), y = S^T C + D x; y silu(z) is RMS-normalised
+    in `norm_groups` equal parts and scaled. Per sequence: S and the
+    convolution's last taps - 1 inputs."""
+
+    kind = "ssd"
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float,
+                 dtype: torch.dtype) -> None:
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        H, DV, N = spec.heads, spec.vdim or spec.dim, spec.state or spec.dim
+        G = spec.groups or 1
+        if H % G:
+            raise ValueError("heads must be a multiple of groups")
+        self.H, self.DV, self.N, self.G = H, DV, N, G
+        self.D = N
+        self.K = max(int(spec.conv), 1)
+        inner = H * DV
+        if inner % max(spec.norm_groups, 1):
+            raise ValueError("norm_groups must divide heads * vdim")
+        self.inner = inner
+        self.C = inner + 2 * G * N        # convolved channels x | B | C
+        self.in_proj = nn.Parameter(
+            torch.empty(inner + self.C + H, width, dtype=dtype))
+        self.conv_w = nn.Parameter(
+            torch.empty(self.C, self.K, dtype=torch.float32))
+        self.conv_b = nn.Parameter(torch.empty(self.C, dtype=torch.float32))
+        self.dt_bias = nn.Parameter(torch.empty(H, dtype=torch.float32))
+        self.a_log = nn.Parameter(torch.empty(H, dtype=torch.float32))
+        self.d_skip = nn.Parameter(torch.empty(H, dtype=torch.float32))
+        self.out_norm = nn.Parameter(torch.empty(inner, dtype=torch.float32))
+        self.out_weight = nn.Parameter(
+            torch.empty(width, inner, dtype=dtype))
+
+    def cache_shape(self):
+        return ("multi", [("state", self.H, self.N, self.DV),
+                          ("slots", (self.K - 1, self.C), None)])
+
+    def forward_from_proj(self, proj, meta, cache, out=None):
+        H, G, N, inner, C = self.H, self.G, self.N, self.inner, self.C
+        state, conv_state = cache
+        xbc = ops.short_conv_silu(proj[:, inner:inner + C], self.conv_w,
+                                  conv_state, meta.seq_rows,
+                                  bias=self.conv_b)
+        y32 = ops.linear_scan(
+            "ssd", xbc[:, inner + G * N:], xbc[:, inner:inner + G * N],
+            xbc[:, :inner], proj[:, inner + C:inner + C + H],
+            proj[:, :inner], state, meta.seq_rows, H, G, self.eps,
+            p0=self.dt_bias, p1=self.a_log, p2=self.d_skip)
+        y = ops.add_rms_norm32(y32, [], self.out_norm, self.eps, proj.dtype,
+                               max(self.spec.norm_groups, 1))
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+
+
+class MixerPair(nn.Module):
+    """Two mixers side by side on the same input: each half's projected
+    output is RMS-normalised over the model width with its own weight and
+    the result is their mean (fp32). Both input projections are one
+    GEMM."""
+
+    kind = "pair"
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float,
+                 dtype: torch.dtype, max_pos: int) -> None:
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        self.left = build_mixer(width, spec.left, eps, dtype, max_pos)
+        self.right = build_mixer(width, spec.right, eps, dtype, max_pos)
+        self.left_norm = nn.Parameter(torch.empty(width,
+                                                  dtype=torch.float32))
+        self.right_norm = nn.Parameter(torch.empty(width,
+                                                   dtype=torch.float32))
+        self._fused = None
+
+    def cache_shape(self):
+        return ("multi", [self.left.cache_shape(),
+                          self.right.cache_shape()])
+
+    def _apply(self, fn, *a, **kw):
+        self._fused = None
+        return super()._apply(fn, *a, **kw)
+
+    def fuse(self):
+        """[left rows | right rows] of the input projections as one weight
+        (the halves' parameters become views of it) and one bias (zeros
+        where a half has none; None when neither has one)."""
+        parts = list(self.left.in_params()) + list(self.right.in_params())
+        w = torch.cat([p.data for p in parts], dim=0).contiguous()
+        off = 0
+        for p in parts:
+            p.data = w[off:off + p.shape[0]]
+            off += p.shape[0]
+        n_left = sum(p.shape[0] for p in self.left.in_params())
+        bias = None
+        bl, br = self.left.in_bias(), self.right.in_bias()
+        if bl is not None or br is not None:
+            bias = torch.zeros(w.shape[0], dtype=w.dtype, device=w.device)
+            if bl is not None:
+                bias[:n_left] = bl.data
+            if br is not None:
+                bias[n_left:] = br.data
+        self._fused = (w, bias, n_left)
+        return self._fused
+
+    def project(self, o: torch.Tensor) -> torch.Tensor:
+        return o
+
+    def forward(self, h: torch.Tensor, meta, cache, shared: dict,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        w, bias, n_left = self._fused or self.fuse()
+        proj = (torch.addmm(bias, h, w.t()) if bias is not None
+                else gemm_policy.linear(h, w))
+        a = self.left.project(self.left.forward_from_proj(
+            proj[:, :n_left], meta, cache[0], None, shared))
+        b = self.right.project(self.right.forward_from_proj(
+            proj[:, n_left:], meta, cache[1]))
+        return ops.norm_sum32([a, b], [self.left_norm, self.right_norm],
+                              0.5, self.eps)
+
+
 def build_mixer(width: int, spec: MixerSpec, eps: float,
                 dtype: torch.dtype, max_pos: int = 8192) -> nn.Module:
     if spec.kind == "attention":
-        return TalkAttention(width, spec, dtype, eps)
+        return TalkAttention(width, spec, dtype, eps, max_pos)
+    if spec.kind == "gla":
+        return GatedLinearAttention(width, spec, eps, dtype)
+    if spec.kind == "mlstm":
+        return MatrixLSTM(width, spec, eps, dtype)
+    if spec.kind == "ssd":
+        return StateSpaceDuality(width, spec, eps, dtype)
+    if spec.kind == "pair":
+        return MixerPair(width, spec, eps, dtype, max_pos)
     if spec.kind == "latent_attention":
         return LatentAttention(width, spec, dtype, eps, max_pos)
     if spec.kind == "general_delta":

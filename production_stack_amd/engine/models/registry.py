@@ -37,10 +37,19 @@ def _derusun_cls():
     return DerusunForCausalLM
 
 
+def _bipulorn_cls():
+    from production_stack_amd.engine.models.bipulorn import (
+        BipulornForCausalLM,
+    )
+
+    return BipulornForCausalLM
+
+
 MODEL_CLASSES: Dict[str, Callable] = {
     "llama": _llama_cls,
     "nanurax": _nanurax_cls,
     "derusun": _derusun_cls,
+    "bipulorn": _bipulorn_cls,
 }
 
 
@@ -57,13 +66,20 @@ def _derusun_config(path: str) -> ModelConfig:
     return derusun.config_from_dir(path)
 
 
+def _bipulorn_config(path: str) -> ModelConfig:
+    from production_stack_amd.engine.models import bipulorn
+
+    return bipulorn.config_from_dir(path)
+
+
 CONFIG_READERS: Dict[str, Callable[[str], ModelConfig]] = {
     "Nanurax": _nanurax_config,
     "Derusun": _derusun_config,
+    "Bipulorn": _bipulorn_config,
 }
 
 # families whose layers also run in float32 (the Llama path is bf16-only)
-FP32_FAMILIES = {"nanurax", "derusun"}
+FP32_FAMILIES = {"nanurax", "derusun", "bipulorn"}
 
 
 def config_from_dir(path: str) -> ModelConfig:

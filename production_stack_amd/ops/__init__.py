@@ -416,7 +416,7 @@ def fp8_linear_rowwise(xq, sx, w_q, sw):
 # these run the kernels of `_mixops.so` (ops/native.py) for bf16 or float32
 # activations; on CPU tensors the references run.
 # ---------------------------------------------------------------------------
-ACT_KINDS = {"silu": 0, "gelu_tanh": 1, "clamped_swish": 2}
+ACT_KINDS = {"silu": 0, "gelu_tanh": 1, "clamped_swish": 2, "sigmoid": 3}
 
 
 def _mx():
@@ -563,7 +563,8 @@ def depth_mix(hist: torch.Tensor, n: int, weights: torch.Tensor,
 def gated_act(gate: torch.Tensor, up: torch.Tensor, kind: str,
               limit: float = 0.0, out: torch.Tensor = None) -> torch.Tensor:
     """Gated-MLP inner activation on [T, F] views (row-strided allowed):
-    silu | gelu_tanh | clamped_swish (see reference.gated_act)."""
+    silu | gelu_tanh | clamped_swish | sigmoid (see reference.gated_act);
+    out may be up itself."""
     T, F = gate.shape
     assert up.shape == (T, F) and up.dtype == gate.dtype
     if out is None:
@@ -705,10 +706,14 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
 def attn_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
               q_w, k_w, eps: float, vmix, v_first, k_cache: torch.Tensor,
               v_cache: torch.Tensor, slot_mapping: torch.Tensor,
-              heads: int) -> None:
+              heads: int, cos_sin: torch.Tensor = None,
+              positions: torch.Tensor = None, rot_dims: int = 0) -> None:
     """Per-head query/key RMSNorm (weights q_w / k_w fp32 [D], None = no
     norm; q is rewritten in place), value blend (1 - vmix) v + vmix v_first
     when v_first [T, G*DV] is given (vmix a 0-dim fp32 tensor; v is
+    rewritten in place), rotary turn of the first rot_dims entries of every
+    query and key head (cos_sin fp32 [positions, rot_dims/2, 2] as
+    rope_table builds it, positions int32 [T]; interleaved pairs; q is
     rewritten in place), and append of the keys and values to the paged
     caches [NB, G, BS, D|DV]. q/k/v are row-strided views."""
     NB, G, BS, D = k_cache.shape
@@ -721,9 +726,15 @@ def attn_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     if v_first is not None:
         assert v_first.shape == v.shape and v_first.dtype == v.dtype
         assert vmix.dtype == torch.float32 and vmix.numel() == 1
+    if cos_sin is not None:
+        assert rot_dims % 2 == 0 and 0 < rot_dims <= D
+        assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous()
+        assert cos_sin.shape[1:] == (rot_dims // 2, 2)
+        assert positions.dtype == torch.int32 and positions.shape == (T,)
     if not q.is_cuda:
         reference.attn_prep(q, k, v, q_w, k_w, eps, vmix, v_first, k_cache,
-                            v_cache, slot_mapping, H)
+                            v_cache, slot_mapping, H, cos_sin, positions,
+                            rot_dims)
         return
     assert q.dtype == k.dtype == v.dtype == k_cache.dtype == v_cache.dtype
     assert k_cache.is_contiguous() and v_cache.is_contiguous()
@@ -735,14 +746,16 @@ def attn_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         _p(q_w), _p(k_w), _f(eps), _p(vmix if v_first is not None else None),
         _p(v_first), _rows(v_first, "v_first") if v_first is not None else 0,
         _p(k_cache), _p(v_cache), _p(slot_mapping), T, H, G, D, DV, BS,
+        _p(cos_sin), int(cos_sin.shape[0]) if cos_sin is not None else 0,
+        int(rot_dims) if cos_sin is not None else 0, _p(positions),
         _mx_dtype(q.dtype), _stream())
 
 
 def rope_table(max_pos: int, dims: int, base: float,
-               device=None) -> torch.Tensor:
-    """fp32 [max_pos, dims/2, 2] (cos, sin) of position * base^(-2i/dims),
-    angles in fp32."""
-    return reference.rope_table(max_pos, dims, base, device)
+               device=None, factor: float = 1.0) -> torch.Tensor:
+    """fp32 [max_pos, dims/2, 2] (cos, sin) of position * base^(-2i/dims)
+    / factor, correctly rounded (angles formed in float64 on the host)."""
+    return reference.rope_table(max_pos, dims, base, device, factor)
 
 
 def latent_prep(q_lat: torch.Tensor, q: torch.Tensor, dkv: torch.Tensor,
@@ -783,11 +796,12 @@ def latent_prep(q_lat: torch.Tensor, q: torch.Tensor, dkv: torch.Tensor,
 
 
 def short_conv_silu(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor,
-                    seq_rows: torch.Tensor,
-                    out: torch.Tensor = None) -> torch.Tensor:
+                    seq_rows: torch.Tensor, out: torch.Tensor = None,
+                    bias: torch.Tensor = None) -> torch.Tensor:
     """Causal per-channel convolution over time + silu over a ragged batch
     (see reference.short_conv_silu). x [T, C] row-strided view; w fp32
-    [C, K]; state [slots, K-1, C] of x's dtype, updated."""
+    [C, K]; state [slots, K-1, C] of x's dtype, updated; bias: optional
+    fp32 [C]."""
     T, C = x.shape
     K = w.shape[1]
     assert w.dtype == torch.float32 and w.shape == (C, K) and K >= 1
@@ -795,15 +809,18 @@ def short_conv_silu(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor,
     if out is None:
         out = torch.empty((T, C), dtype=x.dtype, device=x.device)
     assert out.shape == (T, C) and out.dtype == x.dtype
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.shape == (C,)
     if not x.is_cuda:
-        out.copy_(reference.short_conv_silu(x, w, state, seq_rows, x.dtype))
+        out.copy_(reference.short_conv_silu(x, w, state, seq_rows, x.dtype,
+                                            bias))
         return out
     _check_seq_rows(seq_rows)
     assert w.is_contiguous() and state.is_contiguous()
     rc = _mx().mx_short_conv_silu(
-        _p(out), _rows(out, "out"), _p(x), _rows(x, "x"), _p(w), _p(state),
-        _p(seq_rows), seq_rows.shape[0], C, K, T, _mx_dtype(x.dtype),
-        _stream())
+        _p(out), _rows(out, "out"), _p(x), _rows(x, "x"), _p(w), _p(bias),
+        _p(state), _p(seq_rows), seq_rows.shape[0], C, K, T,
+        _mx_dtype(x.dtype), _stream())
     if rc != 0:
         raise RuntimeError(f"short_conv_silu: {K} taps are not built (1-8)")
     return out
@@ -893,4 +910,125 @@ def delta_rule(r, k, v, zw, za, g, w0, ab, normw, state, seq_rows,
         _f(eps), _f(decay_scale), _mx_dtype(r.dtype), _stream())
     if rc != 0:
         raise RuntimeError(f"delta_rule: head dim {D} above 256 is not built")
+    return out
+
+
+def norm_sum32(inputs, weights, scale: float, eps: float) -> torch.Tensor:
+    """fp32 [T, W] = scale * sum_i rmsnorm(inputs[i]) * weights[i]: up to
+    four branch outputs [T, W] of one dtype (row-strided views allowed),
+    each divided by its own root mean square over the row and scaled by
+    its fp32 weight [W]."""
+    inputs, weights = list(inputs), list(weights)
+    n = len(inputs)
+    assert 1 <= n <= 4 and len(weights) == n
+    T, W = inputs[0].shape
+    for x, w in zip(inputs, weights):
+        assert x.shape == (T, W) and x.dtype == inputs[0].dtype
+        assert w.dtype == torch.float32 and w.numel() == W
+    if not inputs[0].is_cuda:
+        return reference.norm_sum32(inputs, weights, scale, eps)
+    out = torch.empty((T, W), dtype=torch.float32, device=inputs[0].device)
+    pad = [None] * (4 - n)
+    xs, ws = inputs + pad, weights + pad
+    _mx().mx_norm_sum32(
+        _p(out), n, _p(xs[0]), _p(xs[1]), _p(xs[2]), _p(xs[3]),
+        *[_rows(x, "input") if x is not None else 0 for x in xs],
+        _p(ws[0]), _p(ws[1]), _p(ws[2]), _p(ws[3]), _f(scale), _f(eps), T, W,
+        _mx_dtype(inputs[0].dtype), _stream())
+    return out
+
+
+def post_norm_add_norm32(x32: torch.Tensor, delta: torch.Tensor,
+                         w_post: torch.Tensor, w_next: torch.Tensor,
+                         eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """Sublayer boundary of a stack that normalises a sublayer's output
+    before it joins the residual stream: x32 += rmsnorm(delta) * w_post
+    (fp32 [T, W], in place; delta [T, W] fp32 or the serving dtype,
+    row-strided view allowed), returns rmsnorm(x32) * w_next in out_dtype:
+    the next sublayer's input. Weights fp32 [W]."""
+    T, W = x32.shape
+    assert x32.dtype == torch.float32 and x32.is_contiguous()
+    assert delta.shape == (T, W)
+    for w in (w_post, w_next):
+        assert w.dtype == torch.float32 and w.numel() == W
+    if not x32.is_cuda:
+        return reference.post_norm_add_norm32(x32, delta, w_post, w_next,
+                                              eps, out_dtype)
+    h = torch.empty((T, W), dtype=out_dtype, device=x32.device)
+    _mx().mx_post_norm_add_norm32(
+        _p(h), _p(x32), _p(delta), _rows(delta, "delta"),
+        _mx_dtype(delta.dtype), _p(w_post), _p(w_next), _f(eps), T, W,
+        _mx_dtype(out_dtype), _stream())
+    return h
+
+
+SCAN_MODES = {"gla": 0, "ssd": 1, "mlstm": 2}
+
+
+def linear_scan(mode: str, q, k, v, dec, gate, state, seq_rows, heads: int,
+                groups: int, eps: float, qscale: float = 1.0,
+                c0: float = 1.0, wr=None, p0=None, p1=None, p2=None,
+                normw=None, aux=None, out=None) -> torch.Tensor:
+    """Gated linear recurrences S <- diag(a) S + w k v^T, o = S^T q over a
+    ragged batch (see reference.linear_scan for the three decay laws and
+    read-outs: "gla" one decay per key channel, "ssd" one per head with a
+    step size and a skip term, "mlstm" exponential gates with a running
+    maximum and a normaliser). q/k [T, G*D], v/gate [T, H*DV], dec
+    [T, H*D] (gla) or [T, H], wr [T, H] (mlstm): row-strided views of one
+    dtype; p0/p1/p2/normw fp32; state fp32 [slots, H, D, DV] and aux fp32
+    [slots, H, D+1] (mlstm) are updated in place. Returns [T, H*DV], fp32
+    for "ssd" (a grouped norm follows), else the inputs' dtype."""
+    T = q.shape[0]
+    H, G = heads, groups
+    D = q.shape[1] // G
+    DV = v.shape[1] // H
+    assert H % G == 0 and q.shape == (T, G * D) and k.shape == (T, G * D)
+    assert v.shape == (T, H * DV) and gate.shape == (T, H * DV)
+    assert state.dtype == torch.float32 and state.shape[1:] == (H, D, DV)
+    dt = q.dtype
+    for t in (k, v, dec, gate):
+        assert t.dtype == dt
+    if mode == "gla":
+        assert dec.shape == (T, H * D) and G == H
+        assert p0.numel() == H * D and normw.numel() == DV
+    elif mode == "ssd":
+        assert dec.shape == (T, H)
+        assert p0.numel() == H and p1.numel() == H and p2.numel() == H
+    elif mode == "mlstm":
+        assert dec.shape == (T, H) and wr.shape == (T, H) and G == H
+        assert wr.dtype == dt
+        assert p0.numel() == H and p1.numel() == H
+        assert normw.numel() == H * DV
+        assert aux.dtype == torch.float32 and aux.shape[1:] == (H, D + 1)
+        assert aux.shape[0] == state.shape[0]
+    else:
+        raise ValueError(f"unknown scan mode {mode!r}")
+    for t in (p0, p1, p2, normw):
+        assert t is None or t.dtype == torch.float32
+    odt = torch.float32 if mode == "ssd" else dt
+    if out is None:
+        out = torch.empty((T, H * DV), dtype=odt, device=q.device)
+    assert out.shape == (T, H * DV) and out.dtype == odt
+    if not q.is_cuda:
+        y = reference.linear_scan(
+            mode, q.reshape(T, G, D), k.reshape(T, G, D),
+            v.reshape(T, H, DV),
+            dec.reshape(T, H, D) if mode == "gla" else dec, wr,
+            gate.reshape(T, H, DV), p0, p1, p2, normw, state, aux, seq_rows,
+            H, G, eps, qscale, c0, dt)
+        out.copy_(y.reshape(T, H * DV))
+        return out
+    _check_seq_rows(seq_rows)
+    assert state.is_contiguous() and (aux is None or aux.is_contiguous())
+    rc = _mx().mx_linear_scan(
+        SCAN_MODES[mode], _p(out), _rows(out, "out"), _p(q), _rows(q, "q"),
+        _p(k), _rows(k, "k"), _p(v), _rows(v, "v"), _p(dec),
+        _rows(dec, "dec"), _p(wr), _rows(wr, "wr") if wr is not None else 0,
+        _p(gate), _rows(gate, "gate"), _p(p0), _p(p1), _p(p2), _p(normw),
+        _p(state), _p(aux), _p(seq_rows), seq_rows.shape[0], H, G, D, DV,
+        _f(eps), _f(qscale), _f(c0), _mx_dtype(dt), _stream())
+    if rc != 0:
+        raise RuntimeError(
+            f"linear_scan: state {D}x{DV} per head is not built (key dims "
+            "up to 256, value dims up to 1023)")
     return out

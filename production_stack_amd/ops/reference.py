@@ -263,7 +263,8 @@ def depth_mix(hist, n: int, weights, base, delta):
 def gated_act(gate, up, kind: str, limit: float, out_dtype):
     """Gated-MLP inner activation, fp32 math, one rounding at the end.
     silu: silu(g)*u; gelu_tanh: gelu_tanh(g)*u; clamped_swish:
-    g' = min(g, limit), u' = clamp(u, +-limit), g' sigmoid(1.702 g') (u'+1).
+    g' = min(g, limit), u' = clamp(u, +-limit), g' sigmoid(1.702 g') (u'+1);
+    sigmoid: sigmoid(g)*u (an output gate).
     """
     g = gate.float()
     u = up.float()
@@ -275,6 +276,8 @@ def gated_act(gate, up, kind: str, limit: float, out_dtype):
         g = torch.clamp(g, max=limit)
         u = torch.clamp(u, min=-limit, max=limit)
         y = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+    elif kind == "sigmoid":
+        y = torch.sigmoid(g) * u
     else:
         raise ValueError(kind)
     return y.to(out_dtype)
@@ -342,23 +345,33 @@ def talk_attention(q, k_cache, v_cache, block_tables, token_seq, token_pos,
 
 
 def attn_prep(q, k, v, q_w, k_w, eps: float, vmix, v_first, k_cache,
-              v_cache, slot_mapping, heads: int):
+              v_cache, slot_mapping, heads: int, cos_sin=None,
+              positions=None, rot_dims: int = 0):
     """Query/key head norm, value blend and cache append of one attention
     layer. q [T, H*D] is normalised in place per head (x / rms(x) * q_w,
     fp32 math); k [T, G*D] likewise with k_w and appended; v [T, G*DV]
     becomes (1 - vmix) v + vmix v_first when v_first is given (vmix a
     0-dim fp32 tensor), is written back, and appended. q_w / k_w None:
-    no norm."""
+    no norm. With cos_sin (fp32 [positions, rot_dims/2, 2]) the first
+    rot_dims entries of every query and key head turn by the row of the
+    token's position (interleaved pairs), after the norm."""
     T = q.shape[0]
     G, bs, D = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     DV = v_cache.shape[3]
-    if q_w is not None:
+    cs = cos_sin[positions.long()][:, None] if cos_sin is not None else None
+    if q_w is not None or cs is not None:
         qf = q.float().view(T, heads, D)
-        qf = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * q_w
-        q.copy_(qf.view(T, heads * D).to(q.dtype))
+        if q_w is not None:
+            qf = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True)
+                                  + eps) * q_w
+        if cs is not None:
+            qf = _rotate(qf, cs, rot_dims)
+        q.copy_(qf.reshape(T, heads * D).to(q.dtype))
     kf = k.float().view(T, G, D)
     if k_w is not None:
         kf = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) * k_w
+    if cs is not None:
+        kf = _rotate(kf, cs, rot_dims)
     vf = v.float()
     if v_first is not None:
         lam = vmix.float()
@@ -367,13 +380,17 @@ def attn_prep(q, k, v, q_w, k_w, eps: float, vmix, v_first, k_cache,
     kv_append(kf, vf.view(T, G, DV), k_cache, v_cache, slot_mapping)
 
 
-def rope_table(max_pos: int, dims: int, base: float, device=None):
-    """fp32 [max_pos, dims/2, 2] = (cos, sin) of position * base^(-2i/dims)."""
-    i = torch.arange(0, dims, 2, dtype=torch.float32, device=device)
-    f = torch.pow(torch.tensor(float(base), dtype=torch.float32,
-                               device=device), -i / dims)
-    a = torch.arange(max_pos, dtype=torch.float32, device=device)[:, None] * f
-    return torch.stack([torch.cos(a), torch.sin(a)], dim=-1).contiguous()
+def rope_table(max_pos: int, dims: int, base: float, device=None,
+               factor: float = 1.0):
+    """fp32 [max_pos, dims/2, 2] = (cos, sin) of position * base^(-2i/dims)
+    / factor (linear position scaling). The angles are formed in float64 on
+    the host, so an entry is the correctly rounded fp32 value."""
+    i = torch.arange(0, dims, 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                  -i / dims) / float(factor)
+    a = torch.arange(max_pos, dtype=torch.float64)[:, None] * f
+    t = torch.stack([torch.cos(a), torch.sin(a)], dim=-1).float()
+    return t.to(device).contiguous() if device is not None else t.contiguous()
 
 
 def _rotate(x, cs, dims: int):
@@ -414,11 +431,12 @@ def latent_prep(q_lat, q, dkv, norm_w, eps: float, cos_sin, positions,
     return full.reshape(T, H * (L + rot_dim)).to(out_dtype)
 
 
-def short_conv_silu(x, w, state, seq_rows, out_dtype):
+def short_conv_silu(x, w, state, seq_rows, out_dtype, bias=None):
     """Causal per-channel convolution over time followed by silu. x [T, C];
     w fp32 [C, K] (last column weighs the current token); state
     [slots, K-1, C] holds a sequence's last K-1 inputs (oldest first) and is
-    updated; a segment at position 0 starts from zeros."""
+    updated; a segment at position 0 starts from zeros. bias: optional
+    fp32 [C] added before the silu."""
     T, C = x.shape
     K = w.shape[1]
     y = torch.empty(T, C, dtype=torch.float32)
@@ -426,6 +444,8 @@ def short_conv_silu(x, w, state, seq_rows, out_dtype):
         past = state[slot].float() if p0 > 0 else torch.zeros(K - 1, C)
         ext = torch.cat([past, x[t0:t0 + n].float()], dim=0)   # [K-1+n, C]
         acc = torch.zeros(n, C)
+        if bias is not None:
+            acc = acc + bias.float()
         for j in range(K):
             acc += ext[j:j + n] * w[:, j]
         y[t0:t0 + n] = acc
@@ -509,4 +529,105 @@ def delta_rule(r, k, v, zw, za, g, w0, ab, normw, state, seq_rows,
     var = out.pow(2).mean(-1, keepdim=True)
     y = out * torch.rsqrt(var + eps) * normw.view(1, H, D)
     y = y * torch.sigmoid(g.float())
+    return y.to(out_dtype)
+
+
+def norm_sum32(inputs, weights, scale: float, eps: float):
+    """fp32 [T, W] = scale * sum_i rmsnorm(inputs[i]) * weights[i]."""
+    acc = None
+    for x, w in zip(inputs, weights):
+        xf = x.float()
+        y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w
+        acc = y if acc is None else acc + y
+    return acc * scale
+
+
+def post_norm_add_norm32(x32, delta, w_post, w_next, eps: float, out_dtype):
+    """x32 += rmsnorm(delta) * w_post (fp32, in place); returns
+    rmsnorm(x32) * w_next in out_dtype."""
+    d = delta.float()
+    x32.add_(d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w_post)
+    return (x32 * torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + eps)
+            * w_next).to(out_dtype)
+
+
+def _log_sigmoid(z):
+    return torch.clamp(z, max=0.0) - torch.log1p(torch.exp(-z.abs()))
+
+
+def linear_scan(mode: str, q, k, v, dec, wr, gate, p0, p1, p2, normw, state,
+                aux, seq_rows, heads: int, groups: int, eps: float,
+                qscale: float, c0: float, out_dtype):
+    """Gated linear recurrences S <- diag(a) S + w k v^T, o = S^T q over a
+    ragged batch; S fp32 [slots, H, D, DV] updated in place, a segment at
+    position 0 starts from zeros. q/k [T, G, D] (head h reads group
+    h // (H / G)), v [T, H, DV], gate [T, H, DV].
+    mode "gla": dec [T, H, D] raw, a = sigmoid(dec + p0)^c0 per key channel,
+      w = 1, q *= qscale; result rmsnorm_DV(o) * normw[DV] * silu(gate).
+    mode "ssd": dec [T, H] raw, dt = softplus(dec + p0[h]),
+      a = exp(-exp(p1[h]) dt), w = dt; result (o + p2[h] v) * silu(gate),
+      fp32.
+    mode "mlstm": dec / wr [T, H] raw forget / input gates; f =
+      logsigmoid(cap(dec + p1[h])), i = cap(wr + p0[h]), cap(z) = c0
+      tanh(z / c0); running maximum m (aux[slot, h, D]) and normaliser n
+      (aux[slot, h, :D]): m' = max(f + m, i), a = exp(f + m - m'), w =
+      exp(i - m'), n <- a n + w k; o / (max(|n.q|, exp(-m')) + 1e-6),
+      q *= qscale; result o / rms_DV(o) * normw[h, DV] * sigmoid(gate)."""
+    T, G, D = q.shape
+    H = heads
+    DV = v.shape[2]
+    rep = H // G
+    qf = q.float().repeat_interleave(rep, dim=1) * qscale
+    kf = k.float().repeat_interleave(rep, dim=1)
+    vf = v.float()
+    if mode == "gla":
+        a_all = torch.exp(_log_sigmoid(dec.float() + p0.view(1, H, D)) * c0)
+        w_all = torch.ones(T, H)
+    elif mode == "ssd":
+        dt = torch.nn.functional.softplus(dec.float() + p0.view(1, H),
+                                          threshold=20.0)
+        a_all = torch.exp(-torch.exp(p1.float()).view(1, H) * dt)
+        w_all = dt
+    elif mode == "mlstm":
+        ig = c0 * torch.tanh((wr.float() + p0.view(1, H)) / c0)
+        fg = _log_sigmoid(c0 * torch.tanh((dec.float() + p1.view(1, H)) / c0))
+    else:
+        raise ValueError(mode)
+    out = torch.empty(T, H, DV, dtype=torch.float32)
+    for t0, n, pos0, slot in seq_rows.tolist():
+        S = state[slot]
+        if pos0 == 0:
+            S.zero_()
+            if aux is not None:
+                aux[slot].zero_()
+        for t in range(t0, t0 + n):
+            if mode == "mlstm":
+                nv, m = aux[slot, :, :D], aux[slot, :, D]
+                m_new = torch.maximum(fg[t] + m, ig[t])
+                a = torch.exp(fg[t] + m - m_new)
+                w = torch.exp(ig[t] - m_new)
+                S.mul_(a.view(H, 1, 1))
+                S.add_((w.view(H, 1) * kf[t]).unsqueeze(-1)
+                       * vf[t].unsqueeze(1))
+                nv.mul_(a.view(H, 1)).add_(w.view(H, 1) * kf[t])
+                m.copy_(m_new)
+                num = torch.einsum("hij,hi->hj", S, qf[t])
+                den = torch.maximum((nv * qf[t]).sum(-1).abs(),
+                                    torch.exp(-m_new)) + 1e-6
+                out[t] = num / den.unsqueeze(-1)
+                continue
+            a = a_all[t]
+            S.mul_(a.unsqueeze(-1) if mode == "gla" else a.view(H, 1, 1))
+            S.add_((w_all[t].view(H, 1) * kf[t]).unsqueeze(-1)
+                   * vf[t].unsqueeze(1))
+            out[t] = torch.einsum("hij,hi->hj", S, qf[t])
+    g = gate.float()
+    if mode == "ssd":
+        y = (out + p2.float().view(1, H, 1) * vf) * g * torch.sigmoid(g)
+        return y
+    y = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps)
+    if mode == "gla":
+        y = y * normw.view(1, 1, DV) * g * torch.sigmoid(g)
+    else:
+        y = y * normw.view(1, H, DV) * torch.sigmoid(g)
     return y.to(out_dtype)
