@@ -1,6 +1,7 @@
 // Per-token preparation kernels of the attention and recurrent mixers:
-//   attn_prep        per-head query/key RMSNorm, value blend with another
-//                    layer's values, paged K/V append;
+//   attn_prep        per-head query/key RMSNorm, rotary turn of the heads'
+//                    leading entries, value blend with another layer's
+//                    values, paged K/V append;
 //   latent_prep      latent RMSNorm, rotary turn of the shared key part and
 //                    of the queries' rotary parts, paged append of
 //                    [latent | key part], assembly of the latent-space
@@ -11,7 +12,11 @@
 // rounding.
 #include "mix_common.h"
 
-// One wave per head: x / sqrt(mean(x^2) + eps) * w over D entries.
+// One wave per head: x / sqrt(mean(x^2) + eps) * w over D entries, then the
+// first rot_dims entries turn in interleaved pairs (2i, 2i+1) by row
+// `position` of the table cs [table_rows][rot_dims / 2][cos, sin]. A lane
+// reads its own entry and its pair partner's (a neighbouring lane's) before
+// it stores, and the wave runs in step, so the query is rewritten in place.
 template <typename T>
 __global__ __launch_bounds__(256) void attn_prep_kernel(
     T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk,
@@ -19,10 +24,14 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
     const float* __restrict__ kw, float eps, const float* __restrict__ vmix,
     const T* __restrict__ vfirst, int ldvf, T* __restrict__ kc,
     T* __restrict__ vc, const int64_t* __restrict__ slots, int H, int G,
-    int D, int DV, int BS) {
+    int D, int DV, int BS, const float* __restrict__ cs, int table_rows,
+    int rot_dims, const int* __restrict__ positions) {
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
+  const float* csr = nullptr;
+  if (cs != nullptr)
+    csr = cs + (size_t)min(max(positions[t], 0), table_rows - 1) * rot_dims;
   const int64_t slot = slots[t];
   const int64_t blk = slot >= 0 ? slot / BS : 0;
   const int off = slot >= 0 ? (int)(slot % BS) : 0;
@@ -42,17 +51,23 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
       ss = mx_wave_sum(ss);
       inv = 1.0f / sqrtf(ss / (float)D + eps);
     }
+    T* dst = nullptr;
     if (is_q) {
-      if (wgt != nullptr) {
-        T* dst = q + (size_t)t * ldq + hh * D;
-        for (int d = lane; d < D; d += 64)
-          MxElem<T>::st(dst + d, MxElem<T>::ld(src + d) * inv * wgt[d]);
-      }
+      if (wgt != nullptr || csr != nullptr) dst = q + (size_t)t * ldq + hh * D;
     } else if (slot >= 0) {
-      T* dst = kc + ((blk * G + g) * BS + off) * (int64_t)D;
+      dst = kc + ((blk * G + g) * BS + off) * (int64_t)D;
+    }
+    if (dst != nullptr) {
       for (int d = lane; d < D; d += 64) {
-        const float x = MxElem<T>::ld(src + d);
-        MxElem<T>::st(dst + d, wgt != nullptr ? x * inv * wgt[d] : x);
+        float x = MxElem<T>::ld(src + d);
+        if (wgt != nullptr) x *= inv * wgt[d];
+        if (csr != nullptr && d < rot_dims) {
+          float y = MxElem<T>::ld(src + (d ^ 1));
+          if (wgt != nullptr) y *= inv * wgt[d ^ 1];
+          const float* e = csr + (d & ~1);
+          x = (d & 1) ? x * e[0] + y * e[1] : x * e[0] - y * e[1];
+        }
+        MxElem<T>::st(dst + d, x);
       }
     }
   }
@@ -145,8 +160,8 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
 template <typename T, int K>
 __global__ __launch_bounds__(256) void short_conv_silu_kernel(
     T* __restrict__ y, int ldy, const T* __restrict__ x, int ldx,
-    const float* __restrict__ w, T* __restrict__ state,
-    const int* __restrict__ seq_rows, int C) {
+    const float* __restrict__ w, const float* __restrict__ bias,
+    T* __restrict__ state, const int* __restrict__ seq_rows, int C) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   const int* sr = seq_rows + 4 * blockIdx.y;
   const int t0 = sr[0], n = sr[1], p0 = sr[2], slot = sr[3];
@@ -157,6 +172,7 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(
   float wk[K], win[P], old[P];
 #pragma unroll
   for (int j = 0; j < K; ++j) wk[j] = w[(size_t)c * K + j];
+  const float b0 = bias != nullptr ? bias[c] : 0.f;
   T* st = state + (size_t)slot * (K - 1) * C;
 #pragma unroll
   for (int j = 0; j < K - 1; ++j) {
@@ -169,7 +185,7 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(
   }
   for (int t = a; t < b; ++t) {
     const float cur = MxElem<T>::ld(x + (size_t)(t0 + t) * ldx + c);
-    float acc = wk[K - 1] * cur;
+    float acc = b0 + wk[K - 1] * cur;
 #pragma unroll
     for (int j = 0; j < K - 1; ++j) acc += wk[j] * win[j];
 #pragma unroll
@@ -202,14 +218,17 @@ void mx_attn_prep(void* q, int ldq, const void* k, int ldk, void* v, int ldv,
                   const void* qw, const void* kw, float eps, const void* vmix,
                   const void* vfirst, int ldvf, void* kc, void* vc,
                   const void* slots, int T_, int H, int G, int D, int DV,
-                  int BS, int dtype, void* stream) {
+                  int BS, const void* cos_sin, int table_rows, int rot_dims,
+                  const void* positions, int dtype, void* stream) {
   if (T_ <= 0) return;
   MX_DISPATCH_DTYPE(dtype, {
     hipLaunchKernelGGL((attn_prep_kernel<T>), dim3(T_), dim3(256), 0,
                        (hipStream_t)stream, (T*)q, ldq, (const T*)k, ldk,
                        (T*)v, ldv, (const float*)qw, (const float*)kw, eps,
                        (const float*)vmix, (const T*)vfirst, ldvf, (T*)kc,
-                       (T*)vc, (const int64_t*)slots, H, G, D, DV, BS);
+                       (T*)vc, (const int64_t*)slots, H, G, D, DV, BS,
+                       (const float*)cos_sin, table_rows, rot_dims,
+                       (const int*)positions);
   })
 }
 
@@ -235,11 +254,13 @@ void mx_latent_prep(void* qf, const void* qlat, const void* q, int ldq,
   case KK:                                                                   \
     hipLaunchKernelGGL((short_conv_silu_kernel<T, KK>), grid, dim3(256), 0,  \
                        (hipStream_t)stream, (T*)y, ldy, (const T*)x, ldx,    \
-                       (const float*)w, (T*)state, (const int*)seq_rows, C); \
+                       (const float*)w, (const float*)bias, (T*)state,       \
+                       (const int*)seq_rows, C);                             \
     break;
 
 int mx_short_conv_silu(void* y, int ldy, const void* x, int ldx,
-                       const void* w, void* state, const void* seq_rows,
+                       const void* w, const void* bias, void* state,
+                       const void* seq_rows,
                        int S_, int C, int K, int T_, int dtype,
                        void* stream) {
   if (S_ <= 0 || T_ <= 0) return 0;

@@ -127,11 +127,12 @@ __global__ __launch_bounds__(256) void depth_mix_kernel(
 #define MX_ACT_SILU 0
 #define MX_ACT_GELU_TANH 1
 #define MX_ACT_CLAMPED_SWISH 2
+#define MX_ACT_SIGMOID 3  // sigmoid(g) * u: an output gate
 
 template <typename T, int KIND>
 __global__ __launch_bounds__(256) void gated_act_kernel(
-    T* __restrict__ out, int ldo, const T* __restrict__ gate, int ldg,
-    const T* __restrict__ up, int ldu, int F, float limit) {
+    T* out, int ldo, const T* __restrict__ gate, int ldg, const T* up,
+    int ldu, int F, float limit) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= F) return;
@@ -143,6 +144,8 @@ __global__ __launch_bounds__(256) void gated_act_kernel(
   } else if (KIND == MX_ACT_GELU_TANH) {
     const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
     y = 0.5f * g * (1.0f + tanhf(z)) * u;
+  } else if (KIND == MX_ACT_SIGMOID) {
+    y = mx_sigmoid(g) * u;
   } else {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
@@ -155,9 +158,8 @@ __global__ __launch_bounds__(256) void gated_act_kernel(
 // checked widths, strides and pointers for alignment.
 template <int KIND>
 __global__ __launch_bounds__(256) void gated_act_bf16x8_kernel(
-    unsigned short* __restrict__ out, int ldo,
-    const unsigned short* __restrict__ gate, int ldg,
-    const unsigned short* __restrict__ up, int ldu, int F, float limit) {
+    unsigned short* out, int ldo, const unsigned short* __restrict__ gate,
+    int ldg, const unsigned short* up, int ldu, int F, float limit) {
   const int t = blockIdx.y;
   const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (c >= F) return;
@@ -178,6 +180,8 @@ __global__ __launch_bounds__(256) void gated_act_bf16x8_kernel(
       } else if (KIND == MX_ACT_GELU_TANH) {
         const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
         y[e] = 0.5f * g * (1.0f + tanhf(z)) * u;
+      } else if (KIND == MX_ACT_SIGMOID) {
+        y[e] = mx_sigmoid(g) * u;
       } else {
         g = fminf(g, limit);
         u = fminf(fmaxf(u, -limit), limit);
@@ -209,6 +213,74 @@ __global__ __launch_bounds__(256) void kv_append_kernel(
     const int g = c / DV, d = c % DV;
     vc[((blk * G + g) * BS + off) * (int64_t)DV + d] = v[(size_t)t * ldv + c];
   }
+}
+
+// out[t] = scale * sum_i x_i[t] / rms(x_i[t]) * w_i  (fp32), up to four
+// inputs of one element type: branch outputs that are normalised one by one
+// before they are averaged.
+template <typename T>
+__global__ __launch_bounds__(256) void norm_sum32_kernel(
+    float* __restrict__ out, int n, const T* __restrict__ x0,
+    const T* __restrict__ x1, const T* __restrict__ x2,
+    const T* __restrict__ x3, int ld0, int ld1, int ld2, int ld3,
+    const float* __restrict__ w0, const float* __restrict__ w1,
+    const float* __restrict__ w2, const float* __restrict__ w3, float scale,
+    float eps, int W) {
+  __shared__ float red[17];
+  __shared__ float sinv[4];
+  const int t = blockIdx.x;
+  const T* xs[4] = {x0 + (size_t)t * ld0, x1 + (size_t)t * ld1,
+                    x2 + (size_t)t * ld2, x3 + (size_t)t * ld3};
+  const float* ws[4] = {w0, w1, w2, w3};
+  for (int i = 0; i < n; ++i) {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+      const float v = MxElem<T>::ld(xs[i] + c);
+      ss += v * v;
+    }
+    ss = mx_block_sum(ss, red);
+    if (threadIdx.x == 0) sinv[i] = 1.0f / sqrtf(ss / (float)W + eps);
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float acc = 0.f;
+    for (int i = 0; i < n; ++i)
+      acc += MxElem<T>::ld(xs[i] + c) * sinv[i] * ws[i][c];
+    out[(size_t)t * W + c] = acc * scale;
+  }
+}
+
+// Sublayer boundary of a stack that normalises a sublayer's output before it
+// joins the stream: x[t] += d[t] / rms(d[t]) * wpost, then
+// h[t] = x[t] / rms(x[t]) * wnext. TD is the element type of the sublayer
+// output (fp32 for fp32 sums of experts), T of the next sublayer's input.
+// Every thread revisits the entries it wrote itself.
+template <typename TD, typename T>
+__global__ __launch_bounds__(256) void post_norm_add_norm32_kernel(
+    T* __restrict__ h, float* __restrict__ x, const TD* __restrict__ d,
+    int ldd, const float* __restrict__ wpost, const float* __restrict__ wnext,
+    float eps, int W) {
+  __shared__ float red[17];
+  const int t = blockIdx.x;
+  const TD* dr = d + (size_t)t * ldd;
+  float* xr = x + (size_t)t * W;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = MxElem<TD>::ld(dr + c);
+    ss += v * v;
+  }
+  ss = mx_block_sum(ss, red);
+  const float dinv = 1.0f / sqrtf(ss / (float)W + eps);
+  float sx = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = xr[c] + MxElem<TD>::ld(dr + c) * dinv * wpost[c];
+    xr[c] = v;
+    sx += v * v;
+  }
+  sx = mx_block_sum(sx, red);
+  const float xinv = 1.0f / sqrtf(sx / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x)
+    MxElem<T>::st(h + (size_t)t * W + c, xr[c] * xinv * wnext[c]);
 }
 
 extern "C" {
@@ -291,6 +363,10 @@ void mx_gated_act(void* out, int ldo, const void* gate, int ldg,
       hipLaunchKernelGGL((gated_act_bf16x8_kernel<MX_ACT_GELU_TANH>), grid8,
                          dim3(256), 0, (hipStream_t)stream, (U*)out, ldo,
                          (const U*)gate, ldg, (const U*)up, ldu, F, limit);
+    } else if (kind == MX_ACT_SIGMOID) {
+      hipLaunchKernelGGL((gated_act_bf16x8_kernel<MX_ACT_SIGMOID>), grid8,
+                         dim3(256), 0, (hipStream_t)stream, (U*)out, ldo,
+                         (const U*)gate, ldg, (const U*)up, ldu, F, limit);
     } else {
       hipLaunchKernelGGL((gated_act_bf16x8_kernel<MX_ACT_CLAMPED_SWISH>),
                          grid8, dim3(256), 0, (hipStream_t)stream, (U*)out,
@@ -307,6 +383,10 @@ void mx_gated_act(void* out, int ldo, const void* gate, int ldg,
                          (const T*)gate, ldg, (const T*)up, ldu, F, limit);
     } else if (kind == MX_ACT_GELU_TANH) {
       hipLaunchKernelGGL((gated_act_kernel<T, MX_ACT_GELU_TANH>), grid,
+                         dim3(256), 0, (hipStream_t)stream, (T*)out, ldo,
+                         (const T*)gate, ldg, (const T*)up, ldu, F, limit);
+    } else if (kind == MX_ACT_SIGMOID) {
+      hipLaunchKernelGGL((gated_act_kernel<T, MX_ACT_SIGMOID>), grid,
                          dim3(256), 0, (hipStream_t)stream, (T*)out, ldo,
                          (const T*)gate, ldg, (const T*)up, ldu, F, limit);
     } else {
@@ -326,6 +406,41 @@ void mx_kv_append(const void* k, int ldk, const void* v, int ldv, void* kc,
                        (hipStream_t)stream, (const T*)k, ldk, (const T*)v,
                        ldv, (T*)kc, (T*)vc, (const int64_t*)slots, G, D, DV,
                        BS);
+  })
+}
+
+void mx_norm_sum32(void* out, int n, const void* x0, const void* x1,
+                   const void* x2, const void* x3, int ld0, int ld1, int ld2,
+                   int ld3, const void* w0, const void* w1, const void* w2,
+                   const void* w3, float scale, float eps, int T_, int W,
+                   int dtype, void* stream) {
+  if (T_ <= 0 || n < 1 || n > 4) return;
+  MX_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((norm_sum32_kernel<T>), dim3(T_), dim3(256), 0,
+                       (hipStream_t)stream, (float*)out, n, (const T*)x0,
+                       (const T*)x1, (const T*)x2, (const T*)x3, ld0, ld1,
+                       ld2, ld3, (const float*)w0, (const float*)w1,
+                       (const float*)w2, (const float*)w3, scale, eps, W);
+  })
+}
+
+void mx_post_norm_add_norm32(void* h, void* x, const void* d, int ldd,
+                             int d_dtype, const void* wpost,
+                             const void* wnext, float eps, int T_, int W,
+                             int dtype, void* stream) {
+  if (T_ <= 0) return;
+  MX_DISPATCH_DTYPE(dtype, {
+    if (d_dtype == MX_BF16) {
+      hipLaunchKernelGGL((post_norm_add_norm32_kernel<mx_bf16, T>), dim3(T_),
+                         dim3(256), 0, (hipStream_t)stream, (T*)h, (float*)x,
+                         (const mx_bf16*)d, ldd, (const float*)wpost,
+                         (const float*)wnext, eps, W);
+    } else {
+      hipLaunchKernelGGL((post_norm_add_norm32_kernel<float, T>), dim3(T_),
+                         dim3(256), 0, (hipStream_t)stream, (T*)h, (float*)x,
+                         (const float*)d, ldd, (const float*)wpost,
+                         (const float*)wnext, eps, W);
+    }
   })
 }
 

@@ -1,8 +1,9 @@
 """Builder and loader of the mixer-kernel library (`_mixops.so`).
 
-The fp32-residual / delta-rule / attention kernels (csrc/resid32.hip,
-csrc/delta_rule.hip, csrc/gated_delta.hip, csrc/talk_attention.hip,
-csrc/mixer_prep.hip, csrc/mfma_attention.hip) expose a plain C ABI, so the
+The fp32-residual / delta-rule / linear-scan / attention kernels
+(csrc/resid32.hip, csrc/delta_rule.hip, csrc/gated_delta.hip,
+csrc/linear_scan.hip, csrc/talk_attention.hip, csrc/mixer_prep.hip,
+csrc/mfma_attention.hip) expose a plain C ABI, so the
 library needs hipcc only: no torch headers, seconds-to-minutes to build, and
 a fresh checkout can compile just these files on first use without building
 the large `_C` extension. Launchers receive raw device pointers and the
@@ -40,6 +41,8 @@ UNITS = [
     ("mfma_attention.hip", []),
     ("gated_delta.hip", ["-DMX_ONLY_DTYPE=0"]),
     ("gated_delta.hip", ["-DMX_ONLY_DTYPE=1"]),
+    # one unit per (decay law, element type)
+    *[("linear_scan.hip", [f"-DLS_ONLY={i}"]) for i in range(6)],
 ]
 
 _lib = None
@@ -96,12 +99,13 @@ def load():
         lib = ctypes.CDLL(LIB_PATH)
         for name in ("mx_delta_rule", "mx_talk_attention",
                      "mx_gated_delta", "mx_short_conv_silu",
-                     "mx_mfma_attention"):
+                     "mx_mfma_attention", "mx_linear_scan"):
             getattr(lib, name).restype = ctypes.c_int
         for name in ("mx_embed_scale", "mx_add_rms_norm32",
                      "mx_add_group_norm32", "mx_group_norm_shift",
                      "mx_depth_mix", "mx_gated_act", "mx_kv_append",
-                     "mx_attn_prep", "mx_latent_prep"):
+                     "mx_attn_prep", "mx_latent_prep", "mx_norm_sum32",
+                     "mx_post_norm_add_norm32"):
             getattr(lib, name).restype = None
         _lib = lib
     return _lib
