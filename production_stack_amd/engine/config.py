@@ -585,6 +585,89 @@ ARCHITECTURES.update({
 })
 
 
+def _bipulorn_stack(
+    name: str, width: int, vocab: int, n_layers: int, *, attn_heads: int,
+    attn_kv: int, attn_dim: int, window: int, rot_dims: int,
+    rot_factor: float, ssd_heads: int, ssd_vdim: int, ssd_state: int,
+    ssd_groups: int, ssd_norm_groups: int, conv: int, gla_heads: int,
+    gla_dim: int, gla_vdim: int, decay_rank: int, tau: float,
+    lstm_heads: int, lstm_dim: int, lstm_vdim: int, gate_cap: float,
+    experts: int, identity: int, top: int, expert_ff: int, shared_ff: int,
+    route_scale: float = 1.0, softcap: float = 30.0,
+) -> ModelConfig:
+    """A Bipulorn stack in the repeating order pair (window attention +
+    state-space), gated linear attention, pair, matrix LSTM; sequential
+    sublayers with normalised, channel-scaled outputs, every layer with a
+    routed feed-forward (identity outputs, score correction, gated shared
+    expert)."""
+    specs = []
+    for i in range(n_layers):
+        k = i % 4
+        if k in (0, 2):
+            left = MixerSpec(
+                kind="attention", heads=attn_heads, kv_heads=attn_kv,
+                dim=attn_dim, vdim=attn_dim, scale=attn_dim ** -0.5,
+                window=window, rope=True, rot_dims=rot_dims,
+                rot_base=10000.0, rot_factor=rot_factor, bias=True,
+                out_bias=True, out_gate=True)
+            right = MixerSpec(
+                kind="ssd", heads=ssd_heads, dim=ssd_state, state=ssd_state,
+                vdim=ssd_vdim, groups=ssd_groups,
+                norm_groups=ssd_norm_groups, conv=conv, rope=False)
+            mixer = MixerSpec(kind="pair", heads=attn_heads, dim=attn_dim,
+                              rope=False, left=left, right=right)
+        elif k == 1:
+            mixer = MixerSpec(kind="gla", heads=gla_heads, dim=gla_dim,
+                              vdim=gla_vdim, tau=tau, decay_rank=decay_rank,
+                              rope=False)
+        else:
+            mixer = MixerSpec(kind="mlstm", heads=lstm_heads, dim=lstm_dim,
+                              vdim=lstm_vdim, gate_cap=gate_cap, rope=False)
+        mlp = MlpSpec(
+            kind="moe", ff=expert_ff, act="silu", experts=experts, top=top,
+            score="softmax", renormalize=True, shared_ff=shared_ff,
+            correction=True, identity=identity, route_scale=route_scale,
+            renorm_eps=1e-20)
+        specs.append(LayerSpec(mixer=mixer, mlp=mlp, parallel=False,
+                               post_norm=True, layer_scale=True))
+    return ModelConfig(
+        name=name, family="bipulorn", hidden_size=width,
+        num_layers=n_layers, num_q_heads=attn_heads, num_kv_heads=attn_kv,
+        head_dim=attn_dim, intermediate_size=max(expert_ff, shared_ff),
+        vocab_size=vocab, max_position=8192, layer_specs=specs,
+        logit_softcap=softcap, bos_token_id=0, eos_token_id=-1)
+
+
+ARCHITECTURES.update({
+    # CPU-runnable test config
+    "tiny-bipulorn": _bipulorn_stack(
+        "tiny-bipulorn", 96, 384, 4, attn_heads=6, attn_kv=3, attn_dim=16,
+        window=40, rot_dims=8, rot_factor=2.0, ssd_heads=6, ssd_vdim=16,
+        ssd_state=24, ssd_groups=3, ssd_norm_groups=2, conv=3, gla_heads=3,
+        gla_dim=16, gla_vdim=32, decay_rank=8, tau=8.0, lstm_heads=3,
+        lstm_dim=16, lstm_vdim=32, gate_cap=12.0, experts=5, identity=2,
+        top=2, expert_ff=32, shared_ff=64, route_scale=1.5),
+    # llama-3.2-1b-sized stack (same width, depth and vocab)
+    "bipulorn-1b": _bipulorn_stack(
+        "bipulorn-1b", 2048, 128256, 16, attn_heads=32, attn_kv=8,
+        attn_dim=64, window=1024, rot_dims=64, rot_factor=1.0,
+        ssd_heads=64, ssd_vdim=64, ssd_state=128, ssd_groups=1,
+        ssd_norm_groups=1, conv=4, gla_heads=8, gla_dim=128, gla_vdim=256,
+        decay_rank=16, tau=16.0, lstm_heads=16, lstm_dim=128,
+        lstm_vdim=128, gate_cap=15.0, experts=8, identity=2, top=2,
+        expert_ff=2048, shared_ff=2048),
+    # llama-3-8b-sized layers (width 4096, head dim 128)
+    "bipulorn-8b": _bipulorn_stack(
+        "bipulorn-8b", 4096, 128256, 32, attn_heads=32, attn_kv=8,
+        attn_dim=128, window=2048, rot_dims=128, rot_factor=1.0,
+        ssd_heads=128, ssd_vdim=64, ssd_state=128, ssd_groups=1,
+        ssd_norm_groups=1, conv=4, gla_heads=16, gla_dim=128, gla_vdim=256,
+        decay_rank=16, tau=16.0, lstm_heads=32, lstm_dim=128,
+        lstm_vdim=128, gate_cap=15.0, experts=8, identity=2, top=2,
+        expert_ff=3584, shared_ff=3584),
+})
+
+
 @dataclass
 class CacheConfig:
     block_size: int = 16

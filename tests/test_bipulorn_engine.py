@@ -1,0 +1,474 @@
+"""Bipulorn through the engine: checkpoint folder -> registry -> runner ->
+scheduler / block manager / state slots, against the float64 oracle in
+tests/oracle_bipulorn.py. Every test builds its own small configuration and
+random weights. CPU runs the reference ops; gpu-marked variants run the HIP
+kernels."""
+
+import json
+import os
+
+import pytest
+import torch
+
+import oracle_bipulorn as O
+from bipulorn_util import (TOL, close, gla, make_cfg, make_engine,
+                           make_weights, mlstm, moe, pair, rel_err,
+                           save_checkpoint)
+from production_stack_amd.engine.models import registry
+from production_stack_amd.engine.sampling import SamplingParams
+
+pytestmark = pytest.mark.filterwarnings("ignore::UserWarning")
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+DTYPES = ["float32", "bfloat16"]
+
+# every mixer kind twice with different sizes; key width != value width;
+# windows of 20 and 33 positions; rotary on part of a head and on all of it,
+# with and without position scaling; convolutions of 3 and 4 taps; layers
+# with and without a feed-forward; routers with and without identity outputs
+# and shared expert; pages of 16
+STACK = [
+    (gla(3, 16, 24, 8.0), moe(24, 5, 2, 3, 1.5, 40)),
+    (pair(4, 2, 16, 24, 20, 0.3, 8, 100.0, 2.0, 4, 12, 16, 2, 2, 3), None),
+    (mlstm(2, 16, 24, 10.0), moe(16, 4, 0, 2, 1.0, 0)),
+    (pair(6, 3, 8, 8, 33, 0.4, 8, 10000.0, None, 2, 20, 24, 1, 1, 4),
+     moe(24, 3, 3, 2, 2.5, 24)),
+    (gla(1, 40, 8, 3.0), None),
+    (mlstm(3, 16, 8, 6.0), moe(24, 5, 2, 3, 1.5, 40)),
+]
+VOCAB = 97
+
+
+@pytest.fixture(scope="module")
+def ckpt(tmp_path_factory):
+    cfg = make_cfg(STACK, width=64, vocab=VOCAB)
+    W = make_weights(cfg, seed=6)
+    path = save_checkpoint(tmp_path_factory.mktemp("bp") / "m", cfg, W)
+    return path, cfg, W
+
+
+def tokens(n, seed, vocab=VOCAB):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def replay(eng, rid, toks, sizes):
+    """Feed toks in portions of the given sizes (None = the rest); returns
+    logits at every position."""
+    out, at = [], 0
+    for s in sizes:
+        s = len(toks) - at if s is None else min(s, len(toks) - at)
+        if s <= 0:
+            continue
+        last = at + s == len(toks)
+        out.append(eng.replay_step(
+            [(rid, toks[at:at + s], list(range(s)))],
+            end=[rid] if last else []))
+        at += s
+    assert at == len(toks)
+    return torch.cat(out)
+
+
+# ---------------------------------------------------------------------------
+def test_registry_reads_checkpoint_folder(ckpt):
+    path, cfg, W = ckpt
+    mc = registry.config_from_dir(path)
+    assert mc.family == "bipulorn" and mc.vocab_size == VOCAB
+    assert mc.hidden_size == 64 and len(mc.layer_specs) == len(STACK)
+    assert mc.has_recurrent_state and mc.logit_softcap == 12.0
+    s0, s1, s2, s3 = mc.layer_specs[:4]
+    m0 = s0.mixer
+    assert (m0.kind, m0.heads, m0.dim, m0.vdim, m0.tau) == (
+        "gla", 3, 16, 24, 8.0)
+    assert m0.decay_rank == 6                      # a tensor shape
+    f0 = s0.mlp
+    assert (f0.experts, f0.identity, f0.top, f0.route_scale, f0.shared_ff,
+            f0.correction, f0.score, f0.act) == (
+        5, 2, 3, 1.5, 40, True, "softmax", "silu")
+    assert s0.post_norm and s0.layer_scale and not s0.parallel
+    m1 = s1.mixer
+    assert m1.kind == "pair" and s1.mlp is None
+    a, b = m1.left, m1.right
+    assert (a.kind, a.heads, a.kv_heads, a.dim, a.vdim, a.window, a.scale,
+            a.rot_dims, a.rot_base, a.rot_factor) == (
+        "attention", 4, 2, 16, 24, 20, 0.3, 8, 100.0, 2.0)
+    assert a.rope and a.bias and a.out_bias and a.out_gate and not a.sink
+    assert (b.kind, b.heads, b.vdim, b.state, b.groups, b.norm_groups,
+            b.conv) == ("ssd", 4, 12, 16, 2, 2, 3)
+    assert (s2.mixer.kind, s2.mixer.gate_cap) == ("mlstm", 10.0)
+    assert s2.mlp.identity == 0 and s2.mlp.shared_ff == 0
+    assert s3.mixer.left.rot_factor == 1.0         # no scaling entry
+    assert "bipulorn" in registry.FP32_FAMILIES
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_whole_prompt_and_every_layer(ckpt, device, dtype):
+    path, cfg, W = ckpt
+    toks = tokens(70, 1)
+    layers = []
+    want = O.forward(cfg, W, toks, layers)
+    eng = make_engine(path, dtype, device)
+    seen = {}
+    eng.runner.model.residual_hook = lambda i, x: seen.__setitem__(
+        i, x.detach().clone())
+    got = replay(eng, "a", toks, [None])
+    assert close(got, want, dtype)
+    assert sorted(seen) == list(range(len(STACK)))
+    for i in range(len(STACK)):
+        assert seen[i].dtype == torch.float32     # fp32 residual stream
+        assert close(seen[i], layers[i], dtype), i
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_first_tokens_and_single_token_prompt(ckpt, device, dtype):
+    path, cfg, W = ckpt
+    eng = make_engine(path, dtype, device)
+    for n in (1, 2, 3, 5):
+        toks = tokens(n, 10 + n)
+        want = O.forward(cfg, W, toks)
+        assert close(replay(eng, f"p{n}", toks, [None]), want, dtype)
+        assert close(replay(eng, f"q{n}", toks, [1] * n), want, dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("sizes", [
+    [1] * 90, [2] * 45, [3, 2, 17, 2, 31, 2, None], [19, 1, 1, 1, None],
+    [20, 20, 13, None], [33, 1, 33, None], [16, 16, 16, 16, 16, None]])
+def test_portions_match_whole_prompt(ckpt, device, dtype, sizes):
+    """Prefill against token-by-token decoding, and portions of several
+    sizes down to two tokens, cut inside pages, windows and scan tiles and
+    exactly on their edges (windows of 20 and 33 positions, pages of 16,
+    tiles of 16 tokens, convolutions of 3 and 4 taps reaching back over a
+    cut)."""
+    path, cfg, W = ckpt
+    toks = tokens(90, 2)
+    want = O.forward(cfg, W, toks)
+    eng = make_engine(path, dtype, device)
+    assert close(replay(eng, "a", toks, sizes), want, dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decode_past_many_windows(ckpt, device):
+    path, cfg, W = ckpt
+    toks = tokens(260, 3)
+    want = O.forward(cfg, W, toks)
+    eng = make_engine(path, "float32", device)
+    got = replay(eng, "a", toks, [37] + [1] * 223)
+    assert rel_err(got, want) < TOL["float32"]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_mixed_batches_reuse_pages_and_slots(ckpt, device, dtype):
+    """Up to three live requests of unequal length per step, portions
+    beside single tokens; the pool (3 slots, 12 pages) is smaller than the
+    sum of all requests, so pages and slots (recurrent states, normaliser
+    and maximum, convolution tail) pass from finished requests to new ones.
+    Every request must equal itself alone."""
+    path, cfg, W = ckpt
+    lens = {"a": 61, "b": 5, "c": 40, "d": 1, "e": 47, "f": 22}
+    toks = {k: tokens(n, 30 + i) for i, (k, n) in enumerate(lens.items())}
+    want = {k: O.forward(cfg, W, v) for k, v in toks.items()}
+    eng = make_engine(path, dtype, device, blocks=12, max_seqs=3)
+    plan = [
+        [("a", 17), ("b", 2), ("c", 3)],
+        [("a", 1), ("b", 3), ("c", 16)],          # b ends
+        [("a", 2), ("d", 1), ("c", 1)],           # d: one-token request
+        [("c", 20), ("e", 31)],                   # a sits out; c ends
+        [("a", 41), ("e", 1), ("f", 2)],          # a ends
+        [("e", 15), ("f", 20)],                   # both end
+    ]
+    at = {k: 0 for k in toks}
+    got = {k: [] for k in toks}
+    for step in plan:
+        entries, end = [], []
+        for rid, n in step:
+            lo = at[rid]
+            entries.append((rid, toks[rid][lo:lo + n], list(range(n))))
+            at[rid] += n
+            if at[rid] == lens[rid]:
+                end.append(rid)
+        out = eng.replay_step(entries, end=end)
+        r0 = 0
+        for rid, n in step:
+            got[rid].append(out[r0:r0 + n])
+            r0 += n
+    assert at == lens
+    bm = eng.block_manager
+    assert bm.num_free == 12 and len(bm.free_slots) == 3   # all given back
+    for k in toks:
+        assert close(torch.cat(got[k]), want[k], dtype), k
+
+
+def oracle_greedy(cfg, W, prompt, n):
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(O.forward(cfg, W, toks)[-1].argmax()))
+    return toks[len(prompt):]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("budget,blocks", [(1 << 20, 64), (7, 64), (24, 9)])
+def test_greedy_generation_through_the_scheduler(ckpt, device, budget,
+                                                 blocks):
+    """LLMEngine.generate: the scheduler's own chunking (token budgets of
+    7 and 24 cut the prompts into portions), continuous batching of three
+    unequal requests, and with 9 pages preemption with recomputation, must
+    all give the oracle's greedy continuation."""
+    path, cfg, W = ckpt
+    prompts = [tokens(45, 50), tokens(3, 51), tokens(28, 52)]
+    n_new = 10
+    want = [oracle_greedy(cfg, W, p, n_new) for p in prompts]
+    eng = make_engine(path, "float32", device, blocks=blocks, max_seqs=3,
+                      budget=budget)
+    out = eng.generate(prompts, SamplingParams(
+        max_tokens=n_new, temperature=0.0, ignore_eos=True))
+    for i in range(3):
+        assert out[f"offline-{i}"] == want[i], i
+    assert eng.block_manager.num_free == blocks
+    assert len(eng.block_manager.free_slots) == 3
+
+
+OTHER_STACKS = [
+    # every mechanism alone, no feed-forward: (stack, width, vocab, eps,
+    # logit cap, decay rank)
+    ([(gla(2, 24, 16, 16.0), None)], 48, 41, 1e-5, 0.0, 4),
+    ([(mlstm(2, 24, 16, 15.0), None)], 48, 41, 1e-5, 5.0, 4),
+    ([(pair(2, 1, 16, 16, 6, 0.25, 16, 50.0, 4.0, 2, 8, 8, 1, 1, 4), None)],
+     32, 41, 1e-6, 0.0, 4),
+    # attention without window and without rotary code, one key/value head
+    # per query head; one convolution tap; groups == heads; one head per
+    # norm group; a router that picks one output; widths no multiple of 8
+    ([(pair(3, 3, 12, 20, 0, 0.3, 0, 1.0, None, 4, 6, 12, 4, 4, 1),
+       moe(20, 3, 1, 1, 1.0, 12)),
+      (gla(5, 12, 20, 1.0), moe(12, 2, 2, 4, 0.5, 0))],
+     72, 53, 3e-4, 30.0, 3),
+    # a window of one position, rotary over the whole head with a large
+    # base, seven taps, a single head in the recurrences, key width above
+    # value width, five query heads on one key/value head
+    ([(mlstm(1, 40, 12, 2.0), moe(16, 6, 0, 2, 3.0, 8)),
+      (pair(5, 1, 20, 12, 1, 0.22, 20, 1e6, 8.0, 1, 24, 40, 1, 3, 7),
+       None),
+      (mlstm(4, 12, 20, 50.0), None)],
+     60, 71, 1e-5, 8.0, 5),
+    # key widths in every padding class of the scan kernel (<= 16, 17-32,
+    # 33-48, above 64), value widths no multiple of the wave's lane groups
+    ([(gla(2, 72, 10, 4.0), None),
+      (mlstm(2, 30, 18, 6.0), None),
+      (pair(2, 2, 8, 8, 5, 0.35, 4, 10.0, 1.0, 3, 10, 70, 1, 2, 2),
+       moe(8, 2, 1, 2, 1.0, 8))],
+     40, 29, 1e-5, 0.0, 2),
+]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", range(len(OTHER_STACKS)))
+def test_other_orders_and_sizes(tmp_path, device, dtype, which):
+    stack, width, vocab, eps, cap, rank = OTHER_STACKS[which]
+    cfg = make_cfg(stack, width=width, vocab=vocab, eps=eps, softcap=cap)
+    W = make_weights(cfg, seed=40 + which, rank=rank)
+    path = save_checkpoint(tmp_path / f"o{which}", cfg, W)
+    toks = tokens(80, 70 + which, vocab=vocab)
+    want = O.forward(cfg, W, toks)
+    eng = make_engine(path, dtype, device)
+    assert close(replay(eng, "a", toks, [None]), want, dtype)
+    assert close(replay(eng, "b", toks, [6, 1, 2, 30, 1, 1, None]), want,
+                 dtype)
+    # two requests side by side, cut differently
+    half = replay_two(eng, toks, [9, 40, None], [33, 2, None])
+    assert close(half[0], want, dtype) and close(half[1], want, dtype)
+
+
+def replay_two(eng, toks, sizes_a, sizes_b):
+    """The same tokens as two requests in shared steps with different
+    cuts; returns both requests' logits at every position."""
+    def cuts(sizes):
+        out, at = [], 0
+        for s in sizes:
+            s = len(toks) - at if s is None else min(s, len(toks) - at)
+            if s > 0:
+                out.append((at, at + s))
+                at += s
+        return out
+    ca, cb = cuts(sizes_a), cuts(sizes_b)
+    got = {"x": [], "y": []}
+    for step in range(max(len(ca), len(cb))):
+        entries, end = [], []
+        for rid, cc in (("x", ca), ("y", cb)):
+            if step < len(cc):
+                a, b = cc[step]
+                entries.append((rid, toks[a:b], list(range(b - a))))
+                if b == len(toks):
+                    end.append(rid)
+        out = eng.replay_step(entries, end=end)
+        r0 = 0
+        for rid, t, _ in entries:
+            got[rid].append(out[r0:r0 + len(t)])
+            r0 += len(t)
+    return torch.cat(got["x"]), torch.cat(got["y"])
+
+
+# ---------------------------------------------------------------------------
+# a key made to stand out, at the window's edges and far away
+# ---------------------------------------------------------------------------
+NEEDLE, PROBE = 3, 4
+
+
+def needle_model(size, rot_dims, width=32, vocab=23):
+    """One pair layer whose attention half lets the PROBE token's query
+    match the NEEDLE token's key far above every other pair (in head
+    entries the rotary code leaves alone), the needle's value being large:
+    whether the needle is visible decides the logits."""
+    stack = [(pair(2, 1, 16, 8, size, 0.5, rot_dims, 100.0, 2.0, 1, 8, 8,
+                   1, 1, 2), None)]
+    cfg = make_cfg(stack, width=width, vocab=vocab, softcap=0.0)
+    W = make_weights(cfg, seed=9)
+    f32 = torch.float32
+    emb = W["embed"].to(f32)
+    emb[:, :2] = 0.0
+    emb[NEEDLE] = 0.0
+    emb[NEEDLE, 0] = 4.0
+    emb[PROBE] = 0.0
+    emb[PROBE, 1] = 4.0
+    W["embed"] = emb.to(torch.bfloat16)
+    W["l0.norm1"] = torch.zeros(width, dtype=torch.bfloat16)
+    q, k, v = (W[f"l0.mix.left.{n}"].to(f32) for n in "qkv")
+    q[:, 1] = 0.0
+    k[:, 0] = 0.0
+    q[15::16, 1] = 6.0          # last entry of every query head
+    k[15::16, 0] = 6.0          # last entry of the key head
+    v[:, 0] = 3.0
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        W[f"l0.mix.left.{n}"] = t.to(torch.bfloat16)
+    # the recurrent half must not carry the needle past the window
+    W["l0.mix.right.in"] = torch.zeros_like(W["l0.mix.right.in"])
+    return cfg, W
+
+
+def needle_tokens(n, needle_at, probe_at, seed, vocab=23):
+    g = torch.Generator().manual_seed(seed)
+    t = torch.randint(5, vocab, (n,), generator=g).tolist()
+    t[needle_at] = NEEDLE
+    t[probe_at] = PROBE
+    return t
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_window_edges_with_a_stand_out_key(tmp_path, device, dtype):
+    """The probe sits at position 99; the needle just inside the window of
+    24 (position 76), just outside (75), on both sides of a page border
+    (79 / 80) and, without a window, far back (position 2). Prompt portions
+    and single decoded tokens both have to see exactly what the oracle
+    sees."""
+    for size, spots in ((24, (76, 75, 79, 80)), (0, (2, 47))):
+        cfg, W = needle_model(size, 8)
+        path = save_checkpoint(tmp_path / f"n{size}", cfg, W)
+        eng = make_engine(path, dtype, device)
+        seen = []
+        for spot in spots:
+            toks = needle_tokens(104, spot, 99, 60 + spot)
+            want = O.forward(cfg, W, toks)
+            seen.append(want[99])
+            for sizes in ([None], [90] + [1] * 14, [77, 2, 2, None],
+                          [64, 35, 1, None]):
+                got = replay(eng, f"r{spot}", toks, sizes)
+                assert close(got, want, dtype), (size, spot, sizes)
+                assert rel_err(got[99:100], want[99:100]) < (
+                    2e-4 if dtype == "float32" else 5e-2), (size, spot)
+        if size:
+            # the test has teeth: inside and outside differ at the probe
+            assert rel_err(seen[0], seen[1]) > 0.3
+
+
+def test_router_choice_uses_the_correction_and_identity_outputs(tmp_path):
+    """Guards oracle and engine together: the correction moves the choice
+    but not the weights; an identity output returns the input."""
+    stack = [(gla(1, 8, 8, 2.0), moe(8, 2, 2, 2, 1.0, 0))]
+    cfg = make_cfg(stack, width=16, vocab=19, softcap=0.0)
+    W = make_weights(cfg, seed=4)
+    toks = tokens(24, 7, 19)
+    base = O.forward(cfg, W, toks)
+    W2 = dict(W)
+    W2["l0.mlp.correction"] = torch.tensor(
+        [5.0, -5.0, -5.0, 5.0]).to(torch.bfloat16)     # expert 0 + identity
+    W3 = dict(W2)
+    W3["l0.mlp.e1.down"] = torch.zeros_like(W["l0.mlp.e1.down"])
+    moved = O.forward(cfg, W2, toks)
+    assert rel_err(moved, base) > 1e-3
+    assert rel_err(O.forward(cfg, W3, toks), moved) == 0.0   # e1 never runs
+    for k, w in enumerate((W, W2)):
+        path = save_checkpoint(tmp_path / f"r{k}", cfg, w)
+        eng = make_engine(path, "float32", "cpu")
+        got = replay(eng, "a", toks, [7, 1, None])
+        assert rel_err(got, O.forward(cfg, w, toks)) < 2e-4
+
+
+def test_named_config_generates_deterministically():
+    """The named tiny stack: random init, engine entry point, greedy."""
+    from production_stack_amd.engine.config import (CacheConfig,
+                                                    EngineConfig,
+                                                    SchedulerConfig)
+    from production_stack_amd.engine.engine import LLMEngine
+
+    def run(budget):
+        eng = LLMEngine(EngineConfig(
+            model="tiny-bipulorn", dtype="float32", max_model_len=256,
+            enforce_eager=True,
+            cache=CacheConfig(num_gpu_blocks=32, block_size=16),
+            scheduler=SchedulerConfig(max_num_seqs=2,
+                                      max_num_batched_tokens=budget,
+                                      max_prefill_chunk=budget)),
+            device="cpu")
+        return eng.generate(
+            [tokens(30, 1, 300), tokens(4, 2, 300)],
+            SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True))
+
+    a, b = run(256), run(11)
+    assert a == b and all(len(v) == 6 for v in a.values())
+
+
+def test_trace_run_command(ckpt, tmp_path):
+    """bin/trace_run end to end: JSON lines in, 'done' lines and logit
+    files out, pool sized by --max-tokens, requests ended and replaced."""
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    path, cfg, W = ckpt
+    root = os.path.join(os.path.dirname(__file__), "..")
+    ta, tb, tc = tokens(40, 80), tokens(7, 81), tokens(21, 82)
+    steps = [
+        {"step": 0, "entries": [
+            {"id": "a", "tokens": ta[:33], "want": [0, 32]},
+            {"id": "b", "tokens": tb, "want": [6]}], "end": ["b"]},
+        {"step": 1, "entries": [
+            {"id": "a", "tokens": ta[33:34], "want": []}], "end": []},
+        {"step": 2, "entries": [
+            {"id": "c", "tokens": tc, "want": [20]},
+            {"id": "a", "tokens": ta[34:], "want": [5]}],
+         "end": ["a", "c"]},
+    ]
+    out = tmp_path / "out"
+    r = subprocess.run(
+        [sys.executable, os.path.join(root, "bin", "trace_run"), "--model",
+         path, "--dtype", "float32", "--out", str(out), "--max-tokens", "128",
+         "--max-seqs", "2", "--device", "cpu"],
+        input="\n".join(json.dumps(s) for s in steps) + "\n",
+        capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    done = [ln for ln in r.stdout.splitlines() if ln.startswith("done ")]
+    assert done == ["done 0", "done 1", "done 2"]
+    assert not (out / "1.f32").exists()
+    wa, wb, wc = (O.forward(cfg, W, t) for t in (ta, tb, tc))
+    g0 = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4")
+                          .reshape(3, -1).copy())
+    g2 = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4")
+                          .reshape(2, -1).copy())
+    assert rel_err(g0, torch.stack([wa[0], wa[32], wb[6]])) < 2e-4
+    assert rel_err(g2, torch.stack([wc[20], wa[39]])) < 2e-4
