@@ -111,10 +111,14 @@ class User:
 
 
 # --compare-family: prefill / decode throughput of a model family beside the
-# closest Llama config at equal width, depth, dense-ff width and vocabulary
+# closest existing config at equal width, depth and vocabulary (Llama for the
+# first two; for Bipulorn the other hybrid with routed feed-forwards, whose
+# expert widths are the same)
 COMPARE_PAIRS = {
     "nanurax": [("nanurax-1b", "llama-3.2-1b"), ("nanurax-8b", "llama-3-8b")],
     "derusun": [("derusun-1b", "llama-3.2-1b"), ("derusun-8b", "llama-3-8b")],
+    "bipulorn": [("bipulorn-1b", "nanurax-1b"),
+                 ("bipulorn-8b", "nanurax-8b")],
 }
 
 
@@ -225,7 +229,7 @@ def main() -> None:
                     choices=sorted(COMPARE_PAIRS),
                     help="instead of the serving benchmark, measure prefill "
                          "and decode throughput of this family beside the "
-                         "closest Llama config at equal size")
+                         "closest existing config at equal size")
     ap.add_argument("--compare-models", default=None,
                     help="new:base[,new:base] architecture names")
     ap.add_argument("--compare-layers", type=int, default=8)

@@ -1,0 +1,361 @@
+"""The Bipulorn mechanisms one at a time.
+
+CPU part: the reference ops against the float64 oracle's per-mechanism
+functions (tests/oracle_bipulorn.py), fed in ragged portions with stale
+state in the slots. GPU part (marked gpu): every new HIP kernel against the
+PyTorch fp32 reference of the same op, over head sizes of every padding
+class, ragged batches, single tokens and slots that were used before."""
+
+import pytest
+import torch
+
+import oracle_bipulorn as O
+from production_stack_amd import ops
+from production_stack_amd.engine.models.ffn import route
+from production_stack_amd.ops import reference as R
+
+F64 = torch.float64
+
+
+def rnd(g, *shape, scale=1.0):
+    return torch.randn(*shape, generator=g) * scale
+
+
+def segments(lens, pos0s, slots):
+    rows, t0 = [], 0
+    for n, p, s in zip(lens, pos0s, slots):
+        rows.append([t0, n, p, s])
+        t0 += n
+    return torch.tensor(rows, dtype=torch.int32), t0
+
+
+def relerr(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-30))
+
+
+# ---------------------------------------------------------------------------
+# CPU: reference ops in portions against whole-sequence float64 mechanisms
+# ---------------------------------------------------------------------------
+def scan_in_portions(mode, cuts, T, H, G, D, DV, inp, par, eps, qscale, c0,
+                     device="cpu", dtype=torch.float32):
+    """One sequence fed in portions through ops.linear_scan on a slot that
+    holds garbage from an earlier owner."""
+    state = torch.full((3, H, D, DV), 7.0)
+    aux = torch.full((3, H, D + 1), -3.0) if mode == "mlstm" else None
+    mv = lambda t: None if t is None else t.to(device)     # noqa: E731
+    state, aux = mv(state), mv(aux)
+    outs, at = [], 0
+    for n in cuts:
+        sl = slice(at, at + n)
+        sr = torch.tensor([[0, n, at, 1]], dtype=torch.int32)
+        args = {k: (mv(v[sl].to(dtype)) if v is not None else None)
+                for k, v in inp.items()}
+        outs.append(ops.linear_scan(
+            mode, args["q"], args["k"], args["v"], args["dec"], args["gate"],
+            state, mv(sr), H, G, eps, qscale=qscale, c0=c0, wr=args["wr"],
+            p0=mv(par.get("p0")), p1=mv(par.get("p1")), p2=mv(par.get("p2")),
+            normw=mv(par.get("normw")), aux=aux).float().cpu())
+        at += n
+    assert at == T
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("cuts", [[50], [1] * 50, [2] * 25, [17, 1, 30, 2]])
+def test_gla_scan_matches_the_recurrence(cuts):
+    g = torch.Generator().manual_seed(1)
+    T, H, D, DV, tau, eps = 50, 2, 12, 20, 4.0, 1e-5
+    q, k = rnd(g, T, H * D), rnd(g, T, H * D)
+    v, gate, z = rnd(g, T, H * DV), rnd(g, T, H * DV), rnd(g, T, H * D, scale=2)
+    bias, normw = rnd(g, H * D) + 2.0, rnd(g, DV) * 0.2 + 1.0
+    got = scan_in_portions(
+        "gla", cuts, T, H, H, D, DV,
+        dict(q=q, k=k, v=v, dec=z, gate=gate, wr=None),
+        dict(p0=bias, normw=normw), eps, D ** -0.5, 1.0 / tau)
+    # plain recurrence in float64
+    S = torch.zeros(H, D, DV, dtype=F64)
+    want = torch.zeros(T, H, DV, dtype=F64)
+    a = torch.sigmoid((z + bias).to(F64)).pow(1.0 / tau).view(T, H, D)
+    for t in range(T):
+        S = a[t][:, :, None] * S + k[t].to(F64).view(H, D, 1) \
+            * v[t].to(F64).view(H, 1, DV)
+        want[t] = torch.einsum("hdv,hd->hv", S,
+                               q[t].to(F64).view(H, D) * D ** -0.5)
+    want = O.unit_rms(want, eps) * normw.to(F64)
+    want = want.reshape(T, H * DV) * O.silu(gate.to(F64))
+    assert relerr(got, want) < 1e-5
+
+
+@pytest.mark.parametrize("cuts", [[40], [1] * 40, [16, 16, 8], [3, 35, 2]])
+def test_ssd_scan_matches_the_recurrence(cuts):
+    g = torch.Generator().manual_seed(2)
+    T, H, G, N, P = 40, 4, 2, 10, 6
+    B, C = rnd(g, T, G * N), rnd(g, T, G * N)
+    x, z, dt = rnd(g, T, H * P), rnd(g, T, H * P), rnd(g, T, H)
+    dtb, alog, dsk = rnd(g, H), rnd(g, H) * 0.5, rnd(g, H)
+    got = scan_in_portions(
+        "ssd", cuts, T, H, G, N, P,
+        dict(q=C, k=B, v=x, dec=dt, gate=z, wr=None),
+        dict(p0=dtb, p1=alog, p2=dsk), 0.0, 1.0, 1.0)
+    S = torch.zeros(H, N, P, dtype=F64)
+    want = torch.zeros(T, H, P, dtype=F64)
+    step = O.softplus((dt + dtb).to(F64))
+    A = torch.exp(alog.to(F64))
+    for t in range(T):
+        Bt = B[t].to(F64).view(G, N).repeat_interleave(H // G, 0)
+        Ct = C[t].to(F64).view(G, N).repeat_interleave(H // G, 0)
+        xt = x[t].to(F64).view(H, P)
+        S = torch.exp(-A * step[t])[:, None, None] * S \
+            + step[t][:, None, None] * Bt[:, :, None] * xt[:, None, :]
+        want[t] = torch.einsum("hnp,hn->hp", S, Ct) \
+            + dsk.to(F64)[:, None] * xt
+    want = want.reshape(T, H * P) * O.silu(z.to(F64))
+    assert relerr(got, want) < 1e-5
+
+
+@pytest.mark.parametrize("cuts", [[60], [1] * 60, [16, 1, 16, 27], [2] * 30])
+@pytest.mark.parametrize("cap,gain", [(15.0, 1.0), (3.0, 4.0)])
+def test_mlstm_scan_matches_the_recurrence(cuts, cap, gain):
+    """gain 4 with cap 3 drives both gates into the cap; the running
+    maximum starts at 0, so early tokens are bounded by exp(-m), later ones
+    by |n.q|."""
+    g = torch.Generator().manual_seed(3)
+    T, H, D, DV, eps = 60, 2, 10, 14, 1e-5
+    q, k = rnd(g, T, H * D), rnd(g, T, H * D)
+    v, gate = rnd(g, T, H * DV), rnd(g, T, H * DV)
+    zi, zf = rnd(g, T, H, scale=gain), rnd(g, T, H, scale=gain)
+    bi, bf = rnd(g, H), rnd(g, H) + 2.0
+    normw = rnd(g, H * DV) * 0.2 + 1.0
+    got = scan_in_portions(
+        "mlstm", cuts, T, H, H, D, DV,
+        dict(q=q, k=k, v=v, dec=zf, gate=gate, wr=zi),
+        dict(p0=bi, p1=bf, normw=normw), eps, D ** -0.5, cap)
+    ig = cap * torch.tanh((zi + bi).to(F64) / cap)
+    fg = torch.nn.functional.logsigmoid(
+        cap * torch.tanh((zf + bf).to(F64) / cap))
+    S = torch.zeros(H, D, DV, dtype=F64)
+    n = torch.zeros(H, D, dtype=F64)
+    m = torch.zeros(H, dtype=F64)
+    want = torch.zeros(T, H, DV, dtype=F64)
+    bounded_by_m = 0
+    for t in range(T):
+        m2 = torch.maximum(fg[t] + m, ig[t])
+        a, b = torch.exp(fg[t] + m - m2), torch.exp(ig[t] - m2)
+        kt, qt = k[t].to(F64).view(H, D), q[t].to(F64).view(H, D) * D ** -0.5
+        S = a[:, None, None] * S + b[:, None, None] * kt[:, :, None] \
+            * v[t].to(F64).view(H, 1, DV)
+        n = a[:, None] * n + b[:, None] * kt
+        m = m2
+        nq = (n * qt).sum(-1).abs()
+        bounded_by_m += int((nq < torch.exp(-m)).sum())
+        want[t] = torch.einsum("hdv,hd->hv", S, qt) / (
+            torch.maximum(nq, torch.exp(-m)) + 1e-6)[:, None]
+    assert 0 < bounded_by_m < T * H          # both branches of the bound
+    want = O.unit_rms(want, eps).reshape(T, H * DV) * normw.to(F64)
+    want = want * torch.sigmoid(gate.to(F64))
+    assert relerr(got, want) < 1e-5
+
+
+def test_conv_bias_and_state_over_cuts():
+    g = torch.Generator().manual_seed(4)
+    T, C, K = 23, 10, 4
+    x, w, b = rnd(g, T, C), rnd(g, C, K), rnd(g, C)
+    want = O.causal_conv_silu(x.to(F64), w.to(F64), b.to(F64))
+    state = torch.full((2, K - 1, C), 9.0)
+    outs, at = [], 0
+    for n in (1, 2, 1, 7, 12):
+        sr = torch.tensor([[0, n, at, 1]], dtype=torch.int32)
+        outs.append(ops.short_conv_silu(x[at:at + n], w, state, sr, bias=b))
+        at += n
+    assert relerr(torch.cat(outs), want) < 1e-6
+
+
+def test_rotary_prep_matches_interleaved_pairs():
+    g = torch.Generator().manual_seed(5)
+    T, H, G, D, DV, dims = 9, 4, 2, 12, 6, 8
+    q, k, v = rnd(g, T, H * D), rnd(g, T, G * D), rnd(g, T, G * DV)
+    pos = torch.tensor([0, 1, 2, 700, 701, 5, 6, 7, 4000], dtype=torch.int32)
+    kc = torch.zeros(2, G, 16, D)
+    vc = torch.zeros(2, G, 16, DV)
+    slots = torch.arange(T, dtype=torch.long) + 3
+    table = ops.rope_table(4096, dims, 10000.0, None, 4.0)
+    q_in = q.clone()
+    ops.attn_prep(q, k, v, None, None, 1e-5, None, None, kc, vc, slots, H,
+                  cos_sin=table, positions=pos, rot_dims=dims)
+    want_q = O.rotary(q_in.to(F64).view(T, H, D), pos, dims, 10000.0, 4.0)
+    want_k = O.rotary(k.to(F64).view(T, G, D), pos, dims, 10000.0, 4.0)
+    assert relerr(q.view(T, H, D), want_q) < 1e-6
+    got_k = kc.view(2, G, 16, D).permute(0, 2, 1, 3).reshape(32, G, D)[3:3 + T]
+    assert relerr(got_k, want_k) < 1e-6
+    # entries past the rotated ones pass unchanged
+    assert torch.equal(q.view(T, H, D)[..., dims:],
+                       q_in.view(T, H, D)[..., dims:])
+
+
+def test_router_scores_choice_and_weights():
+    g = torch.Generator().manual_seed(6)
+    T, W, n_out, top = 40, 16, 7, 3
+    x, rw = rnd(g, T, W), rnd(g, n_out, W)
+    corr = rnd(g, n_out) * 0.3
+    w, sel = route(x, rw, top, "softmax", True, corr, 2.5, 1e-20)
+    s = torch.softmax(x.to(F64) @ rw.to(F64).t(), -1)
+    want_sel = torch.topk(s + corr.to(F64), top, dim=-1).indices
+    assert torch.equal(sel.sort(-1).values, want_sel.sort(-1).values)
+    # the correction changed some choices but never the weights
+    assert not torch.equal(want_sel.sort(-1).values,
+                           torch.topk(s, top, -1).indices.sort(-1).values)
+    ws = s.gather(-1, sel)
+    assert relerr(w, ws / ws.sum(-1, keepdim=True) * 2.5) < 1e-5
+
+
+def test_branch_norms_and_sublayer_boundary():
+    g = torch.Generator().manual_seed(7)
+    T, W, eps = 5, 24, 1e-4
+    a, b = rnd(g, T, W), rnd(g, T, W) * 30.0
+    wa, wb = rnd(g, W), rnd(g, W)
+    got = ops.norm_sum32([a, b], [wa, wb], 0.5, eps)
+    want = 0.5 * (O.norm_plain(a.to(F64), wa, eps)
+                  + O.norm_plain(b.to(F64), wb, eps))
+    assert relerr(got, want) < 1e-6
+    x, d = rnd(g, T, W), rnd(g, T, W) * 0.01
+    wp, wn = rnd(g, W), rnd(g, W)
+    x64 = x.to(F64) + O.norm_plain(d.to(F64), wp, eps)
+    h = ops.post_norm_add_norm32(x, d, wp, wn, eps, torch.float32)
+    assert relerr(x, x64) < 1e-6               # the stream, updated in place
+    assert relerr(h, O.norm_plain(x64, wn, eps)) < 1e-6
+
+
+# ---------------------------------------------------------------------------
+# GPU: HIP kernels against the reference ops
+# ---------------------------------------------------------------------------
+GPU_DTYPES = [torch.float32, torch.bfloat16]
+
+
+def scan_case(mode, H, G, D, DV, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    # ragged batch: a long portion that starts a sequence, one that goes
+    # on, single tokens of both kinds, a two-token portion
+    sr, T = segments([37, 18, 1, 1, 2], [0, 40, 0, 9, 5], [2, 0, 4, 1, 3])
+    inp = dict(q=rnd(g, T, G * D), k=rnd(g, T, G * D), v=rnd(g, T, H * DV),
+               gate=rnd(g, T, H * DV), wr=None)
+    par = {}
+    if mode == "gla":
+        inp["dec"] = rnd(g, T, H * D, scale=2.0)
+        par = dict(p0=rnd(g, H * D) + 2.0, normw=rnd(g, DV) * 0.2 + 1.0)
+        c0 = 1.0 / 6.0
+    elif mode == "ssd":
+        inp["dec"] = rnd(g, T, H)
+        par = dict(p0=rnd(g, H), p1=rnd(g, H) * 0.5, p2=rnd(g, H))
+        c0 = 1.0
+    else:
+        inp["dec"] = rnd(g, T, H, scale=2.0)
+        inp["wr"] = rnd(g, T, H, scale=2.0)
+        par = dict(p0=rnd(g, H), p1=rnd(g, H) + 2.0,
+                   normw=rnd(g, H * DV) * 0.2 + 1.0)
+        c0 = 5.0
+    inp = {k: (v.to(dtype) if v is not None else None)
+           for k, v in inp.items()}
+    state = rnd(g, 6, H, D, DV)
+    aux = None
+    if mode == "mlstm":
+        aux = rnd(g, 6, H, D + 1)
+        aux[..., D] = aux[..., D].abs()
+    return sr, inp, par, c0, state, aux
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", GPU_DTYPES)
+@pytest.mark.parametrize("mode", ["gla", "ssd", "mlstm"])
+@pytest.mark.parametrize("H,G,D,DV", [
+    (2, 1, 8, 5), (3, 3, 16, 16), (4, 2, 24, 33), (2, 2, 40, 64),
+    (2, 1, 64, 64), (6, 3, 72, 20), (2, 2, 128, 128), (1, 1, 160, 96),
+    (1, 1, 256, 200), (2, 2, 48, 255)])
+def test_linear_scan_kernel(mode, H, G, D, DV, dtype):
+    if mode != "ssd":
+        G = H
+    sr, inp, par, c0, state, aux = scan_case(mode, H, G, D, DV, dtype, D + DV)
+    eps, qs = 1e-5, D ** -0.5
+    want_state = state.clone()
+    want_aux = aux.clone() if aux is not None else None
+    want = ops.linear_scan(
+        mode, inp["q"], inp["k"], inp["v"], inp["dec"], inp["gate"],
+        want_state, sr, H, G, eps, qscale=qs, c0=c0, wr=inp["wr"],
+        aux=want_aux, **par)
+    dev = "cuda"
+    mv = lambda t: None if t is None else t.to(dev)        # noqa: E731
+    st, ax = state.to(dev), mv(aux)
+    got = ops.linear_scan(
+        mode, mv(inp["q"]), mv(inp["k"]), mv(inp["v"]), mv(inp["dec"]),
+        mv(inp["gate"]), st, sr.to(dev), H, G, eps, qscale=qs, c0=c0,
+        wr=mv(inp["wr"]), aux=ax, **{k: v.to(dev) for k, v in par.items()})
+    tol = 2e-5 if dtype == torch.float32 else 6e-3
+    assert relerr(got, want) < tol
+    # slot 5 belongs to nobody in this batch and must stay as it was
+    assert torch.equal(st[5].cpu(), state[5])
+    assert relerr(st, want_state) < 2e-5
+    if aux is not None:
+        assert relerr(ax, want_aux) < 2e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", GPU_DTYPES)
+@pytest.mark.parametrize("H,G,D,DV,dims", [
+    (4, 2, 12, 6, 8), (8, 4, 64, 128, 32), (3, 1, 20, 8, 20),
+    (2, 2, 130, 16, 64)])
+def test_rotary_prep_kernel(H, G, D, DV, dims, dtype):
+    g = torch.Generator().manual_seed(H + D)
+    T, BS, NB = 21, 16, 4
+    q, k, v = (rnd(g, T, n).to(dtype) for n in (H * D, G * D, G * DV))
+    pos = torch.randint(0, 3000, (T,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(NB * BS, generator=g)[:T]
+    table = ops.rope_table(3000, dims, 10000.0, None, 2.0)
+    kc, vc = torch.zeros(NB, G, BS, D).to(dtype), \
+        torch.zeros(NB, G, BS, DV).to(dtype)
+    q0 = q.clone()
+    ops.attn_prep(q0, k, v, None, None, 1e-5, None, None, kc, vc, slots, H,
+                  cos_sin=table, positions=pos, rot_dims=dims)
+    dq, dk, dv = q.cuda(), k.cuda(), v.cuda()
+    dkc, dvc = torch.zeros_like(kc).cuda(), torch.zeros_like(vc).cuda()
+    ops.attn_prep(dq, dk, dv, None, None, 1e-5, None, None, dkc, dvc,
+                  slots.cuda(), H, cos_sin=table.cuda(),
+                  positions=pos.cuda(), rot_dims=dims)
+    tol = 1e-6 if dtype == torch.float32 else 4e-3
+    assert relerr(dq, q0) < tol and relerr(dkc, kc) < tol
+    assert torch.equal(dvc.cpu(), vc)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", GPU_DTYPES)
+def test_small_kernels(dtype):
+    g = torch.Generator().manual_seed(11)
+    T, W, eps = 19, 200, 1e-5
+    tol = 1e-6 if dtype == torch.float32 else 4e-3
+    a, b = rnd(g, T, W).to(dtype), (rnd(g, T, W) * 20).to(dtype)
+    wa, wb = rnd(g, W), rnd(g, W)
+    want = R.norm_sum32([a, b], [wa, wb], 0.5, eps)
+    got = ops.norm_sum32([a.cuda(), b.cuda()], [wa.cuda(), wb.cuda()], 0.5,
+                         eps)
+    assert got.dtype == torch.float32 and relerr(got, want) < 1e-6
+    for ddt in (dtype, torch.float32):
+        x, d = rnd(g, T, W), rnd(g, T, W).to(ddt)
+        wp, wn = rnd(g, W), rnd(g, W)
+        xd = x.cuda()
+        h = ops.post_norm_add_norm32(xd, d.cuda(), wp.cuda(), wn.cuda(), eps,
+                                     dtype)
+        want_h = R.post_norm_add_norm32(x, d, wp, wn, eps, dtype)
+        assert relerr(xd, x) < 1e-6 and relerr(h, want_h) < tol
+    gate, up = rnd(g, T, 72).to(dtype), rnd(g, T, 72).to(dtype)
+    upd = up.cuda()
+    ops.gated_act(gate.cuda(), upd, "sigmoid", out=upd)          # in place
+    assert relerr(upd, R.gated_act(gate, up, "sigmoid", 0.0, dtype)) < tol
+    # convolution with bias, ragged, stale state
+    C, K = 70, 4
+    sr, Tn = segments([9, 1, 5], [0, 7, 3], [1, 0, 2])
+    x = rnd(g, Tn, C).to(dtype)
+    w, bias = rnd(g, C, K), rnd(g, C)
+    st = rnd(g, 4, K - 1, C).to(dtype)
+    st_d = st.cuda()
+    want = R.short_conv_silu(x, w, st, sr, dtype, bias)
+    got = ops.short_conv_silu(x.cuda(), w.cuda(), st_d, sr.cuda(),
+                              bias=bias.cuda())
+    assert relerr(got, want) < tol and relerr(st_d, st) < 1e-6
