@@ -1,7 +1,8 @@
 """Feed-forward building blocks shared by the model families.
 
   * route():       fp32 router with softmax or sigmoid scores, top-k and
-                   optional renormalisation of the chosen weights;
+                   optional renormalisation of the chosen weights (torch
+                   ops; SparseMoE uses the one-kernel ops.moe_route);
   * sparse_moe():  expert dispatch: rows are sorted by expert once (one
                    host read of the per-expert counts per call) and every
                    expert runs the dense GEMM path over its slice, with the
@@ -184,15 +185,14 @@ class SparseMoE(nn.Module):
     # counts on the host every layer
     DENSE_MAX_ROWS = 128
 
-    def _all_experts(self, x: torch.Tensor, weights: torch.Tensor,
-                     sel: torch.Tensor) -> torch.Tensor:
+    def _all_experts(self, x: torch.Tensor,
+                     wm: torch.Tensor) -> torch.Tensor:
         """Every expert over every row; exact because the experts have no
-        biases: a zero-weighted input (or output) contributes exactly 0."""
+        biases: a zero-weighted input (or output) contributes exactly 0.
+        wm fp32 [T, router outputs]: the routing weights, zero where an
+        output was not chosen."""
         sp = self.spec
         T, E, ff = x.shape[0], sp.experts, sp.ff
-        wm = torch.zeros((T, E + sp.identity), dtype=torch.float32,
-                         device=x.device)
-        wm.scatter_(1, sel, weights)
         w_id = wm[:, E:].sum(dim=1, keepdim=True) if sp.identity else None
         wm = wm[:, :E].t().unsqueeze(-1)                # [E, T, 1]
         if sp.weight_on_input:
@@ -227,12 +227,13 @@ class SparseMoE(nn.Module):
         Returns fp32 [T, width]: several experts' outputs are summed in
         fp32."""
         sp = self.spec
-        weights, sel = route(x, self.router, sp.top, sp.score,
-                             sp.renormalize, self.correction,
-                             sp.route_scale, sp.renorm_eps)
+        # one kernel: logits, scores, choice, weights, dense weight matrix
+        weights, sel, wm = ops.moe_route(
+            x, self.router, sp.top, sp.score, sp.renormalize,
+            self.correction, sp.route_scale, sp.renorm_eps)
         T = x.shape[0]
         if T <= self.DENSE_MAX_ROWS and T * sp.top >= sp.experts:
-            out = self._all_experts(x, weights, sel)
+            out = self._all_experts(x, wm)
         else:
             out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
             sparse_moe(x, weights, sel, sp.experts + sp.identity,

@@ -1032,3 +1032,39 @@ def linear_scan(mode: str, q, k, v, dec, gate, state, seq_rows, heads: int,
             f"linear_scan: state {D}x{DV} per head is not built (key dims "
             "up to 256, value dims up to 1023)")
     return out
+
+
+def moe_route(x: torch.Tensor, router_w: torch.Tensor, top: int,
+              score: str = "softmax", renormalize: bool = True,
+              correction: torch.Tensor = None, scale: float = 1.0,
+              renorm_eps: float = 0.0):
+    """Router of a routed feed-forward in one kernel (see
+    reference.moe_route): fp32 logits of x [T, W] against router_w
+    [n_out, W] (both of the serving dtype), softmax or sigmoid scores, the
+    `top` best by score + correction (fp32 [n_out], softmax only), weights
+    = chosen scores / (sum + renorm_eps) when renormalize, times scale.
+    Returns (weights fp32 [T, top], indices int64 [T, top], dense fp32
+    [T, n_out] with the weights at the chosen outputs and zeros
+    elsewhere)."""
+    T, W = x.shape
+    n_out = router_w.shape[0]
+    assert router_w.shape == (n_out, W) and router_w.dtype == x.dtype
+    assert score in ("softmax", "sigmoid") and 1 <= top <= n_out
+    if correction is not None:
+        assert score == "softmax" and correction.dtype == torch.float32
+        assert correction.shape == (n_out,)
+    if not x.is_cuda:
+        return reference.moe_route(x, router_w, top, score, renormalize,
+                                   correction, scale, renorm_eps)
+    assert router_w.is_contiguous()
+    sel = torch.empty((T, top), dtype=torch.long, device=x.device)
+    wts = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    dense = torch.empty((T, n_out), dtype=torch.float32, device=x.device)
+    rc = _mx().mx_moe_route(
+        _p(sel), _p(wts), _p(dense), _p(x), _rows(x, "x"), _p(router_w),
+        _p(correction), T, W, n_out, int(top), int(score == "sigmoid"),
+        int(bool(renormalize)), _f(renorm_eps), _f(scale),
+        _mx_dtype(x.dtype), _stream())
+    if rc != 0:
+        raise RuntimeError(f"moe_route: {n_out} router outputs exceed 1024")
+    return wts, sel, dense

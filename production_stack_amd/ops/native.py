@@ -3,7 +3,7 @@
 The fp32-residual / delta-rule / linear-scan / attention kernels
 (csrc/resid32.hip, csrc/delta_rule.hip, csrc/gated_delta.hip,
 csrc/linear_scan.hip, csrc/talk_attention.hip, csrc/mixer_prep.hip,
-csrc/mfma_attention.hip) expose a plain C ABI, so the
+csrc/mfma_attention.hip, csrc/moe_route.hip) expose a plain C ABI, so the
 library needs hipcc only: no torch headers, seconds-to-minutes to build, and
 a fresh checkout can compile just these files on first use without building
 the large `_C` extension. Launchers receive raw device pointers and the
@@ -39,6 +39,7 @@ UNITS = [
     ("delta_rule.hip", ["-DMX_ONLY_DTYPE=1"]),
     ("mixer_prep.hip", []),
     ("mfma_attention.hip", []),
+    ("moe_route.hip", []),
     ("gated_delta.hip", ["-DMX_ONLY_DTYPE=0"]),
     ("gated_delta.hip", ["-DMX_ONLY_DTYPE=1"]),
     # one unit per (decay law, element type)
@@ -99,7 +100,8 @@ def load():
         lib = ctypes.CDLL(LIB_PATH)
         for name in ("mx_delta_rule", "mx_talk_attention",
                      "mx_gated_delta", "mx_short_conv_silu",
-                     "mx_mfma_attention", "mx_linear_scan"):
+                     "mx_mfma_attention", "mx_linear_scan",
+                     "mx_moe_route"):
             getattr(lib, name).restype = ctypes.c_int
         for name in ("mx_embed_scale", "mx_add_rms_norm32",
                      "mx_add_group_norm32", "mx_group_norm_shift",

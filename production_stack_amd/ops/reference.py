@@ -631,3 +631,26 @@ def linear_scan(mode: str, q, k, v, dec, wr, gate, p0, p1, p2, normw, state,
     else:
         y = y * normw.view(1, H, DV) * torch.sigmoid(g)
     return y.to(out_dtype)
+
+
+def moe_route(x, router_w, top: int, score: str, renormalize: bool,
+              correction, scale: float, renorm_eps: float):
+    """Router of a routed feed-forward: fp32 logits, softmax | sigmoid
+    scores, the `top` outputs with the largest score + correction (sigmoid
+    scores are ranked by their logits), weights = chosen scores, divided by
+    (their sum + renorm_eps) when renormalize, times scale. Returns
+    (weights [T, top], indices [T, top], dense [T, n_out])."""
+    logits = torch.nn.functional.linear(x.float(), router_w.float())
+    if score == "softmax":
+        probs = torch.softmax(logits, dim=-1)
+        pick = probs + correction if correction is not None else probs
+    else:
+        probs = torch.sigmoid(logits)
+        pick = logits
+    sel = torch.topk(pick, top, dim=-1).indices
+    w = probs.gather(-1, sel)
+    if renormalize:
+        w = w / (w.sum(-1, keepdim=True) + renorm_eps)
+    w = w * scale
+    dense = torch.zeros_like(probs).scatter_(1, sel, w)
+    return w, sel, dense

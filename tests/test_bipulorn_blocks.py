@@ -197,7 +197,12 @@ def test_router_scores_choice_and_weights():
     T, W, n_out, top = 40, 16, 7, 3
     x, rw = rnd(g, T, W), rnd(g, n_out, W)
     corr = rnd(g, n_out) * 0.3
-    w, sel = route(x, rw, top, "softmax", True, corr, 2.5, 1e-20)
+    w, sel, dense = ops.moe_route(x, rw, top, "softmax", True, corr, 2.5,
+                                  1e-20)
+    w2, sel2 = route(x, rw, top, "softmax", True, corr, 2.5, 1e-20)
+    assert torch.equal(sel, sel2) and relerr(w, w2) < 1e-6
+    assert relerr(dense.gather(1, sel), w) == 0.0
+    assert relerr(dense.sum(-1), w.sum(-1)) < 1e-6      # zeros elsewhere
     s = torch.softmax(x.to(F64) @ rw.to(F64).t(), -1)
     want_sel = torch.topk(s + corr.to(F64), top, dim=-1).indices
     assert torch.equal(sel.sort(-1).values, want_sel.sort(-1).values)
@@ -359,3 +364,25 @@ def test_small_kernels(dtype):
     got = ops.short_conv_silu(x.cuda(), w.cuda(), st_d, sr.cuda(),
                               bias=bias.cuda())
     assert relerr(got, want) < tol and relerr(st_d, st) < 1e-6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", GPU_DTYPES)
+@pytest.mark.parametrize("T,W,n_out,top,score,renorm,use_corr", [
+    (1, 64, 5, 1, "softmax", True, True),
+    (37, 200, 7, 3, "softmax", True, True),
+    (300, 96, 20, 4, "softmax", False, False),
+    (65, 128, 130, 9, "softmax", True, True),
+    (50, 72, 6, 2, "sigmoid", False, False),
+    (9, 40, 3, 3, "sigmoid", True, False)])
+def test_router_kernel(T, W, n_out, top, score, renorm, use_corr, dtype):
+    g = torch.Generator().manual_seed(T + n_out)
+    x = rnd(g, T, W).to(dtype)
+    rw = (rnd(g, n_out, W) * 3.0 / W ** 0.5).to(dtype)
+    corr = rnd(g, n_out) * 0.2 if use_corr else None
+    w, sel, dense = R.moe_route(x, rw, top, score, renorm, corr, 1.7, 1e-20)
+    gw, gsel, gdense = ops.moe_route(
+        x.cuda(), rw.cuda(), top, score, renorm,
+        corr.cuda() if use_corr else None, 1.7, 1e-20)
+    assert torch.equal(gsel.cpu(), sel)               # best first, same order
+    assert relerr(gw, w) < 1e-5 and relerr(gdense, dense) < 1e-5
