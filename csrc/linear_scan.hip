@@ -271,12 +271,11 @@ __global__ __launch_bounds__(MAXT) void linear_scan_kernel(
       p2, normw, state, aux, seq_rows, S_, H, G, D, DV, eps, qscale, c0,     \
       stream
 
-template <typename T, typename TO, int MODE, int DKP>
-static int launch_linear_scan(LS_ARGS) {
+// P lanes share a state column. WIDE: only the 1024-thread bound is built
+// (fallback forms are reached with more than 256 columns only).
+template <typename T, typename TO, int MODE, int DKP, int P, bool WIDE>
+static int launch_linear_scan_p(LS_ARGS) {
   constexpr int TILE = DKP <= 128 ? 16 : 8;
-  // lanes per column: enough to keep a lane's rows within 32 registers
-  // where the column count allows it
-  constexpr int P = DKP >= 64 ? 4 : (DKP >= 32 ? 2 : 1);
   const int cols = DV + (MODE == LS_MLSTM ? 1 : 0);
   const int threads = ((cols * P + 63) / 64) * 64;
   if (threads > 1024) return 1;
@@ -295,13 +294,36 @@ static int launch_linear_scan(LS_ARGS) {
       qscale, c0)
   // the launch bound follows the thread count, so small launches keep a
   // lane's rows and the tile's outputs out of scratch
-  if (threads <= 256) {
-    LS_LAUNCH(256);
-  } else {
-    LS_LAUNCH(1024);
+  if constexpr (!WIDE) {
+    if (threads <= 256) {
+      LS_LAUNCH(256);
+      return 0;
+    }
   }
+  LS_LAUNCH(1024);
 #undef LS_LAUNCH
   return 0;
+}
+
+template <typename T, typename TO, int MODE, int DKP>
+static int launch_linear_scan(LS_ARGS) {
+  // lanes per column: enough to keep a lane's rows within 32 registers
+  // where the column count allows it; heads with more value columns than
+  // fit a workgroup that way take fewer lanes per column (more rows, and
+  // scratch, per lane: correct, not fast)
+  constexpr int P0 = DKP >= 64 ? 4 : (DKP >= 32 ? 2 : 1);
+  const int cols = DV + (MODE == LS_MLSTM ? 1 : 0);
+  if (cols * P0 <= 1024)
+    return launch_linear_scan_p<T, TO, MODE, DKP, P0, false>(LS_PASS);
+  if constexpr (P0 >= 4) {
+    if (cols * 2 <= 1024)
+      return launch_linear_scan_p<T, TO, MODE, DKP, 2, true>(LS_PASS);
+  }
+  if constexpr (P0 >= 2) {
+    if (cols <= 1024)
+      return launch_linear_scan_p<T, TO, MODE, DKP, 1, true>(LS_PASS);
+  }
+  return 1;
 }
 
 #define LS_CASE(PAD) \

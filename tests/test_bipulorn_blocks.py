@@ -274,7 +274,8 @@ def scan_case(mode, H, G, D, DV, dtype, seed):
 @pytest.mark.parametrize("H,G,D,DV", [
     (2, 1, 8, 5), (3, 3, 16, 16), (4, 2, 24, 33), (2, 2, 40, 64),
     (2, 1, 64, 64), (6, 3, 72, 20), (2, 2, 128, 128), (1, 1, 160, 96),
-    (1, 1, 256, 200), (2, 2, 48, 255)])
+    (1, 1, 256, 200), (2, 2, 48, 255), (1, 1, 64, 256), (1, 1, 40, 600),
+    (1, 1, 128, 520)])
 def test_linear_scan_kernel(mode, H, G, D, DV, dtype):
     if mode != "ssd":
         G = H
