@@ -185,30 +185,36 @@ class SparseMoE(nn.Module):
     # counts on the host every layer
     DENSE_MAX_ROWS = 128
 
-    def _all_experts(self, x: torch.Tensor,
-                     wm: torch.Tensor) -> torch.Tensor:
+    def _all_experts(self, x: torch.Tensor, wm: torch.Tensor,
+                     shared_y: Optional[torch.Tensor] = None,
+                     shared_gate: Optional[torch.Tensor] = None
+                     ) -> torch.Tensor:
         """Every expert over every row; exact because the experts have no
         biases: a zero-weighted input (or output) contributes exactly 0.
         wm fp32 [T, router outputs]: the routing weights, zero where an
-        output was not chosen."""
+        output was not chosen. With the weight on the experts' outputs, the
+        weighted sum, the identity outputs and the gated shared expert
+        (shared_y [T, W], shared_gate [T, 1] pre-sigmoid) are one kernel."""
         sp = self.spec
         T, E, ff = x.shape[0], sp.experts, sp.ff
-        w_id = wm[:, E:].sum(dim=1, keepdim=True) if sp.identity else None
-        wm = wm[:, :E].t().unsqueeze(-1)                # [E, T, 1]
         if sp.weight_on_input:
-            xe = (x.float().unsqueeze(0) * wm).to(x.dtype)
+            w_id = (wm[:, E:].sum(dim=1, keepdim=True) if sp.identity
+                    else None)
+            we = wm[:, :E].t().unsqueeze(-1)            # [E, T, 1]
+            xe = (x.float().unsqueeze(0) * we).to(x.dtype)
         else:
             xe = x.unsqueeze(0).expand(E, T, x.shape[1])
         gu = torch.bmm(xe, self.experts_gate_up.transpose(1, 2))
         gu2 = gu.view(E * T, 2 * ff)
         act = ops.gated_act(gu2[:, :ff], gu2[:, ff:], sp.act, sp.limit)
         y = torch.bmm(act.view(E, T, ff), self.experts_down.transpose(1, 2))
-        y = y.float()
         if not sp.weight_on_input:
-            y = y * wm
-        y = y.sum(dim=0)
+            return ops.moe_combine(y, wm, x, E, shared_y, shared_gate)
+        y = y.float().sum(dim=0)
         if w_id is not None:
             y += x.float() * w_id
+        if shared_y is not None:
+            y += shared_y.float() * torch.sigmoid(shared_gate.float())
         return y
 
     def _expert(self, e: int, xe: torch.Tensor) -> torch.Tensor:
@@ -232,18 +238,18 @@ class SparseMoE(nn.Module):
             x, self.router, sp.top, sp.score, sp.renormalize,
             self.correction, sp.route_scale, sp.renorm_eps)
         T = x.shape[0]
-        if T <= self.DENSE_MAX_ROWS and T * sp.top >= sp.experts:
-            out = self._all_experts(x, wm)
-        else:
-            out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
-            sparse_moe(x, weights, sel, sp.experts + sp.identity,
-                       self._expert,
-                       weight_on_input=sp.weight_on_input, out=out)
+        y = gate = None
         if self.shared is not None:
             sff = sp.shared_ff
             y = self.shared.forward_from_proj(proj[:, :2 * sff])
-            gate = torch.sigmoid(proj[:, 2 * sff:].float())
-            out += y.float() * gate
+            gate = proj[:, 2 * sff:]
+        if T <= self.DENSE_MAX_ROWS and T * sp.top >= sp.experts:
+            return self._all_experts(x, wm, y, gate)
+        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        sparse_moe(x, weights, sel, sp.experts + sp.identity, self._expert,
+                   weight_on_input=sp.weight_on_input, out=out)
+        if y is not None:
+            out += y.float() * torch.sigmoid(gate.float())
         return out
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:

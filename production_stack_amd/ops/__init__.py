@@ -1068,3 +1068,34 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, top: int,
     if rc != 0:
         raise RuntimeError(f"moe_route: {n_out} router outputs exceed 1024")
     return wts, sel, dense
+
+
+def moe_combine(y: torch.Tensor, dense: torch.Tensor, x: torch.Tensor,
+                experts: int, shared_y: torch.Tensor = None,
+                shared_gate: torch.Tensor = None) -> torch.Tensor:
+    """Weighted sum of the all-experts path in one kernel: y [E, T, W] is
+    every expert's output for every row, dense fp32 [T, n_out] the routing
+    weights (zero = not chosen; outputs from `experts` on are identity
+    outputs that return the input x [T, W]); the shared expert's output
+    shared_y [T, W] joins times sigmoid(shared_gate [T, 1]). Returns fp32
+    [T, W]."""
+    E, T, W = y.shape
+    n_out = dense.shape[1]
+    assert E == experts and n_out >= E and dense.shape == (T, n_out)
+    assert dense.dtype == torch.float32 and x.shape == (T, W)
+    assert x.dtype == y.dtype
+    if shared_y is not None:
+        assert shared_y.shape == (T, W) and shared_gate.shape == (T, 1)
+        assert shared_y.dtype == y.dtype and shared_gate.dtype == y.dtype
+    if not y.is_cuda:
+        return reference.moe_combine(y, dense, x, experts, shared_y,
+                                     shared_gate)
+    assert y.is_contiguous() and dense.is_contiguous()
+    out = torch.empty((T, W), dtype=torch.float32, device=y.device)
+    _mx().mx_moe_combine(
+        _p(out), _p(y), _p(dense), n_out, E, _p(x), _rows(x, "x"),
+        _p(shared_y), _rows(shared_y, "shared_y") if shared_y is not None
+        else 0, _p(shared_gate),
+        _rows(shared_gate, "shared_gate") if shared_gate is not None else 0,
+        T, W, _mx_dtype(y.dtype), _stream())
+    return out

@@ -107,6 +107,7 @@ def load():
                      "mx_add_group_norm32", "mx_group_norm_shift",
                      "mx_depth_mix", "mx_gated_act", "mx_kv_append",
                      "mx_attn_prep", "mx_latent_prep", "mx_norm_sum32",
+                     "mx_moe_combine",
                      "mx_post_norm_add_norm32"):
             getattr(lib, name).restype = None
         _lib = lib

@@ -654,3 +654,14 @@ def moe_route(x, router_w, top: int, score: str, renormalize: bool,
     w = w * scale
     dense = torch.zeros_like(probs).scatter_(1, sel, w)
     return w, sel, dense
+
+
+def moe_combine(y, dense, x, experts: int, shared_y=None, shared_gate=None):
+    """fp32 [T, W] = sum_e dense[:, e] y[e] over the experts + (sum of the
+    identity outputs' weights) x + sigmoid(shared_gate) shared_y."""
+    out = torch.einsum("te,etw->tw", dense[:, :experts], y.float())
+    if dense.shape[1] > experts:
+        out = out + dense[:, experts:].sum(-1, keepdim=True) * x.float()
+    if shared_y is not None:
+        out = out + torch.sigmoid(shared_gate.float()) * shared_y.float()
+    return out

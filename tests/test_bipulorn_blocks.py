@@ -387,3 +387,40 @@ def test_router_kernel(T, W, n_out, top, score, renorm, use_corr, dtype):
         corr.cuda() if use_corr else None, 1.7, 1e-20)
     assert torch.equal(gsel.cpu(), sel)               # best first, same order
     assert relerr(gw, w) < 1e-5 and relerr(gdense, dense) < 1e-5
+
+
+def test_combine_weights_identity_and_shared():
+    g = torch.Generator().manual_seed(8)
+    E, n_out, T, W = 3, 5, 7, 12
+    y, x = rnd(g, E, T, W), rnd(g, T, W)
+    dense = torch.zeros(T, n_out)
+    dense[torch.arange(T), torch.arange(T) % n_out] = 0.7
+    dense[torch.arange(T), (torch.arange(T) + 2) % n_out] = 0.4
+    ys, sg = rnd(g, T, W), rnd(g, T, 1)
+    want = torch.zeros(T, W, dtype=F64)
+    for t in range(T):
+        for e in range(n_out):
+            src = y[e, t] if e < E else x[t]
+            want[t] += float(dense[t, e]) * src.to(F64)
+        want[t] += torch.sigmoid(sg[t].to(F64)) * ys[t].to(F64)
+    assert relerr(ops.moe_combine(y, dense, x, E, ys, sg), want) < 1e-6
+    assert relerr(ops.moe_combine(y, dense, x, E) + torch.sigmoid(sg) * ys,
+                  want) < 1e-6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", GPU_DTYPES)
+@pytest.mark.parametrize("E,n_out,T,W,shared", [
+    (8, 10, 64, 520, True), (3, 3, 5, 72, False), (2, 6, 128, 200, True)])
+def test_combine_kernel(E, n_out, T, W, shared, dtype):
+    g = torch.Generator().manual_seed(E + T)
+    y, x = rnd(g, E, T, W).to(dtype), rnd(g, T, W).to(dtype)
+    dense = torch.rand(T, n_out, generator=g)
+    dense[dense < 0.6] = 0.0
+    ys = rnd(g, T, W).to(dtype) if shared else None
+    sg = rnd(g, T, 1).to(dtype) if shared else None
+    want = R.moe_combine(y, dense, x, E, ys, sg)
+    got = ops.moe_combine(y.cuda(), dense.cuda(), x.cuda(), E,
+                          ys.cuda() if shared else None,
+                          sg.cuda() if shared else None)
+    assert got.dtype == torch.float32 and relerr(got, want) < 1e-5
