@@ -192,8 +192,9 @@ class BipulornLayer(nn.Module):
 class BipulornForCausalLM(nn.Module):
     # per-step metadata this family needs from the runner
     needs_seq_meta = True
-    # data-dependent routing keeps decode steps out of hipGraphs
-    supports_decode_graph = False
+    # single-token steps route through the all-experts path (router and
+    # weighted sum are kernels, no host read), so they replay a hipGraph
+    supports_decode_graph = True
 
     def __init__(self, cfg: ModelConfig, tp: int = 1, pp_rank: int = 0,
                  pp_size: int = 1, dtype: torch.dtype = torch.bfloat16
@@ -436,6 +437,9 @@ class BipulornForCausalLM(nn.Module):
         h = ops.add_rms_norm32(x, [], layers[0].norm1, eps, dt)
         shared: dict = {}
         hook = self.residual_hook
+        # steps of single tokens only: every expert over every row
+        dense = True if getattr(meta, "num_prefill_tokens", None) == 0 \
+            else None
         for i, (layer, cache) in enumerate(zip(layers, caches)):
             mx = layer.mixer
             delta, w_post = mx.project(mx(h, meta, cache, shared)), \
@@ -443,7 +447,7 @@ class BipulornForCausalLM(nn.Module):
             if layer.mlp is not None:
                 h = ops.post_norm_add_norm32(x, delta, w_post, layer.norm2,
                                              eps, dt)
-                delta, w_post = layer.mlp(h), layer.post2
+                delta, w_post = layer.mlp(h, dense), layer.post2
             w_next = (layers[i + 1].norm1 if i + 1 < len(layers)
                       else self.final_norm)
             h = ops.post_norm_add_norm32(x, delta, w_post, w_next, eps, dt)

@@ -227,11 +227,13 @@ class SparseMoE(nn.Module):
         return gemm_policy.linear(act, self.experts_down[e])
 
     def forward_from_proj(self, x: torch.Tensor,
-                          proj: Optional[torch.Tensor]) -> torch.Tensor:
+                          proj: Optional[torch.Tensor],
+                          dense: Optional[bool] = None) -> torch.Tensor:
         """x: layer input [T, width]; proj: the shared expert's fused
         projection [T, 2*shared_ff + 1] (None without a shared expert).
-        Returns fp32 [T, width]: several experts' outputs are summed in
-        fp32."""
+        dense=True insists on the all-experts path (no host read: what a
+        captured decode step needs), None picks by batch size. Returns fp32
+        [T, width]: several experts' outputs are summed in fp32."""
         sp = self.spec
         # one kernel: logits, scores, choice, weights, dense weight matrix
         weights, sel, wm = ops.moe_route(
@@ -243,7 +245,9 @@ class SparseMoE(nn.Module):
             sff = sp.shared_ff
             y = self.shared.forward_from_proj(proj[:, :2 * sff])
             gate = proj[:, 2 * sff:]
-        if T <= self.DENSE_MAX_ROWS and T * sp.top >= sp.experts:
+        if dense is None:
+            dense = T <= self.DENSE_MAX_ROWS and T * sp.top >= sp.experts
+        if dense:
             return self._all_experts(x, wm, y, gate)
         out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
         sparse_moe(x, weights, sel, sp.experts + sp.identity, self._expert,
@@ -252,7 +256,8 @@ class SparseMoE(nn.Module):
             out += y.float() * torch.sigmoid(gate.float())
         return out
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor,
+                dense: Optional[bool] = None) -> torch.Tensor:
         proj = (gemm_policy.linear(x, self.fused_in())
                 if self.shared is not None else None)
-        return self.forward_from_proj(x, proj)
+        return self.forward_from_proj(x, proj, dense)

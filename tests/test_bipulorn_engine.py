@@ -472,3 +472,63 @@ def test_trace_run_command(ckpt, tmp_path):
                           .reshape(2, -1).copy())
     assert rel_err(g0, torch.stack([wa[0], wa[32], wb[6]])) < 2e-4
     assert rel_err(g2, torch.stack([wc[20], wa[39]])) < 2e-4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decode_graph_replays_match_eager(ckpt, dtype):
+    """Single-token steps replay a captured hipGraph (padded to a batch
+    bucket, padding rows parked on the spare state slot; the routed
+    feed-forwards take the all-experts path). Three requests of unequal
+    length join and leave, so bucket sizes, padding rows and slots
+    change between replays; eager prompt portions run in between. Every
+    step's logits must match the eager engine's."""
+    from production_stack_amd.engine.config import (CacheConfig,
+                                                    EngineConfig,
+                                                    SchedulerConfig)
+    from production_stack_amd.engine.engine import LLMEngine
+
+    path, cfg, W = ckpt
+
+    def make(eager):
+        return LLMEngine(EngineConfig(
+            model=path, dtype=dtype, max_model_len=256, enforce_eager=eager,
+            cache=CacheConfig(num_gpu_blocks=48, block_size=16,
+                              enable_prefix_caching=False),
+            scheduler=SchedulerConfig(max_num_seqs=4,
+                                      max_num_batched_tokens=64)),
+            device="cuda")
+
+    graph, eager = make(False), make(True)
+    assert graph.runner.graphs is not None and eager.runner.graphs is None
+    prompts = [tokens(37, 90), tokens(5, 91), tokens(70, 92)]
+    lens = [9, 14, 6]
+    outs = []
+    for eng in (graph, eager):
+        got = {}
+        seen = []
+        orig = eng.runner.sample
+
+        def spy(logits, seqs, _orig=orig, _seen=seen):
+            _seen.append(logits.detach().float().cpu().clone())
+            return _orig(logits, seqs)
+
+        eng.runner.sample = spy
+        for i, (p, n) in enumerate(zip(prompts, lens)):
+            eng.add_request(f"r{i}", p, SamplingParams(
+                max_tokens=n, temperature=0.0, ignore_eos=True))
+        while eng.has_unfinished():
+            for o in eng.step():
+                got.setdefault(o.request_id, []).extend(o.new_token_ids)
+        outs.append((got, seen))
+    (g_tok, g_log), (e_tok, e_log) = outs
+    assert len(g_log) == len(e_log) and len(g_log) >= max(lens)
+    if dtype == "float32":
+        assert g_tok == e_tok
+    for a, b in zip(g_log, e_log):
+        assert a.shape == b.shape
+        if dtype == "float32":
+            assert rel_err(a, b) < 2e-4
+    want = [oracle_greedy(cfg, W, p, n) for p, n in zip(prompts, lens)]
+    if dtype == "float32":
+        assert [g_tok[f"r{i}"] for i in range(3)] == want
