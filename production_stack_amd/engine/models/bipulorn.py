@@ -349,7 +349,7 @@ class BipulornForCausalLM(nn.Module):
             param.copy_(t.to(param.dtype))
 
         def unit_offset(param, name):
-            # stored around zero: the norm multiplies by 1 + w
+            # the checkpoint holds the weight's offset from one
             t = f.get_tensor(name)
             check(t, param, name)
             param.copy_(1.0 + t.float())

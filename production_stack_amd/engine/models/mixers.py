@@ -549,7 +549,7 @@ class StateSpaceDuality(_ScanMixer):
 
 
 class MixerPair(nn.Module):
-    """Two mixers side by side on the same input: each half's projected
+    """Two mixers fed the same input: each half's projected
     output is RMS-normalised over the model width with its own weight and
     the result is their mean (fp32). Both input projections are one
     GEMM."""

@@ -32,7 +32,7 @@ def unit_rms(x, eps):
 
 
 def norm_one_plus(x, w, eps):
-    """Stack norm: weight stored around zero."""
+    """Stack norm: the tensor holds the weight minus one."""
     return unit_rms(x, eps) * (1.0 + w.to(F64))
 
 
