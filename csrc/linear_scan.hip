@@ -51,7 +51,8 @@ __global__ __launch_bounds__(MAXT) void linear_scan_kernel(
     const float* __restrict__ p1, const float* __restrict__ p2,
     const float* __restrict__ normw, float* __restrict__ state,
     float* __restrict__ aux, const int* __restrict__ seq_rows, int H, int G,
-    int D, int DV, float eps, float qscale, float c0) {
+    int D, int DV, float eps, float qscale, float c0, int CS, int DVB,
+    float* __restrict__ raw, float* __restrict__ naux) {
   extern __shared__ __align__(16) float lds[];
   constexpr int R = DKP / P;        // rows per lane
   constexpr int RP = P > 1 ? R + 4 : R;
@@ -65,12 +66,18 @@ __global__ __launch_bounds__(MAXT) void linear_scan_kernel(
   float* sem = swr + TILE;          // [TILE] exp(-m)
   float* snq = sem + TILE;          // [TILE] n.q
 
-  const int seg = blockIdx.x / H, hd = blockIdx.x % H;
+  // a head's value columns may be shared out over CS workgroups of DVB
+  // columns each (block cb owns columns cb * DVB ...); every block of a
+  // matrix-LSTM head carries its own copy of the normaliser column
+  const int cb = blockIdx.x % CS, sh = blockIdx.x / CS;
+  const int seg = sh / H, hd = sh % H;
   const int t0 = seq_rows[4 * seg + 0], n = seq_rows[4 * seg + 1];
   const int pos0 = seq_rows[4 * seg + 2], slot = seq_rows[4 * seg + 3];
-  const int j = threadIdx.x / P, p = threadIdx.x % P;
-  const bool vcol = j < DV;                           // a value column
-  const bool ncol = MODE == LS_MLSTM && j == DV;      // the normaliser
+  const int jl = threadIdx.x / P, p = threadIdx.x % P;
+  const int nloc = min(DVB, DV - cb * DVB);           // columns of this block
+  const int j = cb * DVB + jl;
+  const bool vcol = jl < nloc;                        // a value column
+  const bool ncol = MODE == LS_MLSTM && jl == nloc;   // the normaliser
   const bool col = vcol || ncol;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
@@ -83,6 +90,12 @@ __global__ __launch_bounds__(MAXT) void linear_scan_kernel(
   float* Sg = state + ((size_t)slot * H + hd) * (size_t)D * DV;
   float* Ng = MODE == LS_MLSTM ? aux + ((size_t)slot * H + hd) * (D + 1)
                                : nullptr;
+  // Where the new normaliser and maximum go. With shared-out columns the
+  // other workgroups of the head may still have to read the old ones, so
+  // the new ones wait in scratch until the read-out kernel has started.
+  float* Nw = (MODE == LS_MLSTM && naux != nullptr)
+                  ? naux + ((size_t)seg * H + hd) * (D + 1)
+                  : Ng;
   float S[R];  // S[r] = row p + P * r of column j
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -221,6 +234,17 @@ __global__ __launch_bounds__(MAXT) void linear_scan_kernel(
       for (int tt = 0; tt < TILE; ++tt)
         if (tt < nt) o[tt] /= fmaxf(fabsf(snq[tt]), sem[tt]) + 1e-6f;
     }
+    if (raw != nullptr) {
+      // the head's columns are spread over several workgroups: its norm is
+      // taken by the read-out kernel
+      if (vcol && p == 0) {
+#pragma unroll
+        for (int tt = 0; tt < TILE; ++tt)
+          if (tt < nt)
+            raw[(size_t)(t0 + tb + tt) * ((size_t)H * DV) + hv + j] = o[tt];
+      }
+      continue;
+    }
     // per-token sum over the head's value columns of o^2
 #pragma unroll
     for (int tt = 0; tt < TILE; ++tt) {
@@ -252,11 +276,45 @@ __global__ __launch_bounds__(MAXT) void linear_scan_kernel(
       const int i = p + P * r;
       if (i < D) {
         if (vcol) Sg[(size_t)i * DV + j] = S[r];
-        if (ncol) Ng[i] = S[r];
+        if (ncol && cb == 0) Nw[i] = S[r];
       }
     }
   }
-  if (MODE == LS_MLSTM && threadIdx.x == 0) Ng[D] = m_run;
+  if (MODE == LS_MLSTM && threadIdx.x == 0 && cb == 0) Nw[D] = m_run;
+}
+
+// Read-out of heads whose columns were spread over several workgroups: one
+// wave per (token, head): o / rms_DV(o) * weight * gate.
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void scan_readout_kernel(
+    T* __restrict__ out, int ldo, const float* __restrict__ raw,
+    const T* __restrict__ gate, int ldg, const float* __restrict__ normw,
+    int T_, int H, int DV, float eps, const float* __restrict__ naux,
+    float* __restrict__ aux, const int* __restrict__ seq_rows, int S_,
+    int D) {
+  const int w = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (w >= T_ * H) return;
+  if (naux != nullptr && w < S_ * H) {
+    // the matrix LSTM's new normaliser and maximum move into their slot
+    const int slot = seq_rows[4 * (w / H) + 3];
+    const float* src = naux + (size_t)w * (D + 1);
+    float* dst = aux + ((size_t)slot * H + w % H) * (D + 1);
+    for (int c = lane; c <= D; c += 64) dst[c] = src[c];
+  }
+  const int t = w / H, hd = w % H, hv = hd * DV;
+  const float* r = raw + (size_t)t * ((size_t)H * DV) + hv;
+  float ss = 0.f;
+  for (int c = lane; c < DV; c += 64) ss += r[c] * r[c];
+  ss = mx_wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)DV + eps);
+  for (int c = lane; c < DV; c += 64) {
+    const float g = MxElem<T>::ld(gate + (size_t)t * ldg + hv + c);
+    const float y = MODE == LS_GLA
+                        ? r[c] * inv * normw[c] * g * mx_sigmoid(g)
+                        : r[c] * inv * normw[hv + c] * mx_sigmoid(g);
+    MxElem<T>::st(out + (size_t)t * ldo + hv + c, y);
+  }
 }
 
 #define LS_ARGS                                                              \
@@ -265,43 +323,85 @@ __global__ __launch_bounds__(MAXT) void linear_scan_kernel(
       int ldwr, const void *gate, int ldg, const void *p0, const void *p1,   \
       const void *p2, const void *normw, void *state, void *aux,             \
       const void *seq_rows, int S_, int H, int G, int D, int DV, float eps,  \
-      float qscale, float c0, void *stream
+      float qscale, float c0, int T_, void *raw, void *stream
 #define LS_PASS                                                              \
   out, ldo, q, ldq, k, ldk, v, ldv, dec, lddec, wr, ldwr, gate, ldg, p0, p1, \
       p2, normw, state, aux, seq_rows, S_, H, G, D, DV, eps, qscale, c0,     \
-      stream
+      T_, raw, stream
+
+// Key width as the kernels pad it (0: not built).
+static int ls_pad(int D) {
+  const int pads[] = {16, 32, 48, 64, 96, 128, 192, 256};
+  for (int p : pads)
+    if (D <= p) return p;
+  return 0;
+}
+
+// How many workgroups share a head's value columns. A launch of few
+// (segment, head) pairs leaves most of the chip idle and, with wide heads,
+// puts up to 16 waves on one CU's LDS; splitting the columns spreads them
+// over up to 8 CUs as long as every part keeps at least four waves.
+static int ls_splits(int mode, int S_, int H, int D, int DV) {
+  const int dkp = ls_pad(D);
+  if (dkp == 0) return 1;
+  const int P0 = dkp >= 64 ? 4 : (dkp >= 32 ? 2 : 1);
+  if ((DV + (mode == LS_MLSTM ? 1 : 0)) * P0 > 1024) return 1;
+  const long wgs = (long)S_ * H;
+  int cs = 1;
+  while (cs < 8 && wgs * cs * 2 <= 512 && DV % (cs * 2) == 0 &&
+         (DV / (cs * 2)) * P0 >= 256)
+    cs *= 2;
+  return cs;
+}
 
 // P lanes share a state column. WIDE: only the 1024-thread bound is built
 // (fallback forms are reached with more than 256 columns only).
 template <typename T, typename TO, int MODE, int DKP, int P, bool WIDE>
-static int launch_linear_scan_p(LS_ARGS) {
+static int launch_linear_scan_p(LS_ARGS, int CS) {
   constexpr int TILE = DKP <= 128 ? 16 : 8;
-  const int cols = DV + (MODE == LS_MLSTM ? 1 : 0);
+  const int DVB = DV / CS;  // CS divides DV (ls_splits)
+  const int cols = DVB + (MODE == LS_MLSTM ? 1 : 0);
   const int threads = ((cols * P + 63) / 64) * 64;
   if (threads > 1024) return 1;
+  float* rawp = (CS > 1 && MODE != LS_SSD) ? (float*)raw : nullptr;
+  // scratch layout: [T_][H * DV] read-outs, then [S_][H][D + 1]
+  float* nauxp = (rawp != nullptr && MODE == LS_MLSTM)
+                     ? rawp + (size_t)T_ * H * DV
+                     : nullptr;
   const size_t lds =
       (size_t)((MODE == LS_GLA ? 3 : 2) * TILE * (DKP + (P > 1 ? 4 * P : 0)) +
                16 * TILE + 4 * TILE) *
       sizeof(float);
 #define LS_LAUNCH(MAXT)                                                      \
   hipLaunchKernelGGL(                                                        \
-      (linear_scan_kernel<T, TO, MODE, DKP, TILE, P, MAXT>), dim3(S_ * H),   \
-      dim3(threads), lds, (hipStream_t)stream, (TO*)out, ldo, (const T*)q,   \
-      ldq, (const T*)k, ldk, (const T*)v, ldv, (const T*)dec, lddec,         \
-      (const T*)wr, ldwr, (const T*)gate, ldg, (const float*)p0,             \
-      (const float*)p1, (const float*)p2, (const float*)normw,               \
-      (float*)state, (float*)aux, (const int*)seq_rows, H, G, D, DV, eps,    \
-      qscale, c0)
+      (linear_scan_kernel<T, TO, MODE, DKP, TILE, P, MAXT>),                 \
+      dim3(S_ * H * CS), dim3(threads), lds, (hipStream_t)stream, (TO*)out,  \
+      ldo, (const T*)q, ldq, (const T*)k, ldk, (const T*)v, ldv,             \
+      (const T*)dec, lddec, (const T*)wr, ldwr, (const T*)gate, ldg,         \
+      (const float*)p0, (const float*)p1, (const float*)p2,                  \
+      (const float*)normw, (float*)state, (float*)aux, (const int*)seq_rows, \
+      H, G, D, DV, eps, qscale, c0, CS, DVB, rawp, nauxp)
   // the launch bound follows the thread count, so small launches keep a
   // lane's rows and the tile's outputs out of scratch
-  if constexpr (!WIDE) {
-    if (threads <= 256) {
-      LS_LAUNCH(256);
-      return 0;
+  bool small = false;
+  if constexpr (!WIDE) small = threads <= 256;
+  if (small) {
+    if constexpr (!WIDE) LS_LAUNCH(256);
+  } else {
+    LS_LAUNCH(1024);
+  }
+#undef LS_LAUNCH
+  if constexpr (MODE != LS_SSD) {
+    if (rawp != nullptr) {
+      const long waves = (long)T_ * H;
+      hipLaunchKernelGGL((scan_readout_kernel<T, MODE>),
+                         dim3((unsigned)((waves + 3) / 4)), dim3(256), 0,
+                         (hipStream_t)stream, (T*)out, ldo, rawp,
+                         (const T*)gate, ldg, (const float*)normw, T_, H, DV,
+                         eps, nauxp, (float*)aux, (const int*)seq_rows, S_,
+                         D);
     }
   }
-  LS_LAUNCH(1024);
-#undef LS_LAUNCH
   return 0;
 }
 
@@ -313,15 +413,20 @@ static int launch_linear_scan(LS_ARGS) {
   // scratch, per lane: correct, not fast)
   constexpr int P0 = DKP >= 64 ? 4 : (DKP >= 32 ? 2 : 1);
   const int cols = DV + (MODE == LS_MLSTM ? 1 : 0);
-  if (cols * P0 <= 1024)
-    return launch_linear_scan_p<T, TO, MODE, DKP, P0, false>(LS_PASS);
+  if (cols * P0 <= 1024) {
+    // without the scratch buffer the read-out norm cannot be split
+    const int CS = (raw != nullptr || MODE == LS_SSD)
+                       ? ls_splits(MODE, S_, H, D, DV)
+                       : 1;
+    return launch_linear_scan_p<T, TO, MODE, DKP, P0, false>(LS_PASS, CS);
+  }
   if constexpr (P0 >= 4) {
     if (cols * 2 <= 1024)
-      return launch_linear_scan_p<T, TO, MODE, DKP, 2, true>(LS_PASS);
+      return launch_linear_scan_p<T, TO, MODE, DKP, 2, true>(LS_PASS, 1);
   }
   if constexpr (P0 >= 2) {
     if (cols <= 1024)
-      return launch_linear_scan_p<T, TO, MODE, DKP, 1, true>(LS_PASS);
+      return launch_linear_scan_p<T, TO, MODE, DKP, 1, true>(LS_PASS, 1);
   }
   return 1;
 }
@@ -385,13 +490,21 @@ LS_UNIT(mx_linear_scan_mlstm_f32) {
 #endif
 
 #if !defined(LS_ONLY) || LS_ONLY == 0
+extern "C" int mx_linear_scan_splits(int mode, int S_, int H, int D,
+                                     int DV) {
+  return ls_splits(mode, S_, H, D, DV);
+}
+
+// raw: fp32 scratch of T_ * H * DV + S_ * H * (D + 1) entries, needed when
+// mx_linear_scan_splits says a head's columns are shared out (ignored
+// otherwise; without it the launch is not split).
 extern "C" int mx_linear_scan(
     int mode, void* out, int ldo, const void* q, int ldq, const void* k,
     int ldk, const void* v, int ldv, const void* dec, int lddec,
     const void* wr, int ldwr, const void* gate, int ldg, const void* p0,
     const void* p1, const void* p2, const void* normw, void* state, void* aux,
     const void* seq_rows, int S_, int H, int G, int D, int DV, float eps,
-    float qscale, float c0, int dtype, void* stream) {
+    float qscale, float c0, int T_, void* raw, int dtype, void* stream) {
   if (S_ <= 0) return 0;
   if (G < 1 || H % G) return 2;
   const bool bf = dtype == MX_BF16;

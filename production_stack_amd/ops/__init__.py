@@ -1020,13 +1020,22 @@ def linear_scan(mode: str, q, k, v, dec, gate, state, seq_rows, heads: int,
         return out
     _check_seq_rows(seq_rows)
     assert state.is_contiguous() and (aux is None or aux.is_contiguous())
+    # few (segment, head) pairs with wide heads: a head's value columns are
+    # shared out over several workgroups and the read-out norm runs as a
+    # second kernel over this fp32 scratch
+    raw = None
+    if mode != "ssd" and _mx().mx_linear_scan_splits(
+            SCAN_MODES[mode], seq_rows.shape[0], H, D, DV) > 1:
+        raw = torch.empty(
+            T * H * DV + seq_rows.shape[0] * H * (D + 1),
+            dtype=torch.float32, device=q.device)
     rc = _mx().mx_linear_scan(
         SCAN_MODES[mode], _p(out), _rows(out, "out"), _p(q), _rows(q, "q"),
         _p(k), _rows(k, "k"), _p(v), _rows(v, "v"), _p(dec),
         _rows(dec, "dec"), _p(wr), _rows(wr, "wr") if wr is not None else 0,
         _p(gate), _rows(gate, "gate"), _p(p0), _p(p1), _p(p2), _p(normw),
         _p(state), _p(aux), _p(seq_rows), seq_rows.shape[0], H, G, D, DV,
-        _f(eps), _f(qscale), _f(c0), _mx_dtype(dt), _stream())
+        _f(eps), _f(qscale), _f(c0), T, _p(raw), _mx_dtype(dt), _stream())
     if rc != 0:
         raise RuntimeError(
             f"linear_scan: state {D}x{DV} per head is not built (key dims "

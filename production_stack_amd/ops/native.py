@@ -101,6 +101,7 @@ def load():
         for name in ("mx_delta_rule", "mx_talk_attention",
                      "mx_gated_delta", "mx_short_conv_silu",
                      "mx_mfma_attention", "mx_linear_scan",
+                     "mx_linear_scan_splits",
                      "mx_moe_route"):
             getattr(lib, name).restype = ctypes.c_int
         for name in ("mx_embed_scale", "mx_add_rms_norm32",
