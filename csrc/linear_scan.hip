@@ -29,6 +29,13 @@
 // then each thread walks the tile's tokens with broadcast LDS reads and no
 // barrier. The running maximum is a sequential scan over the tile by one
 // thread (a handful of scalar operations per token).
+//
+// Wide heads share their value columns out over several workgroups of four
+// waves (columns never interact inside the
+// recurrence; every part of a matrix-LSTM head carries the normaliser column
+// itself). The read-out norm, which spans the head, then runs as a second
+// kernel over an fp32 scratch, and the new normaliser and maximum wait in
+// scratch until then: a part that starts late must still find the old ones.
 #include "mix_common.h"
 
 #define LS_GLA 0
@@ -337,20 +344,21 @@ static int ls_pad(int D) {
   return 0;
 }
 
-// How many workgroups share a head's value columns. A launch of few
-// (segment, head) pairs leaves most of the chip idle and, with wide heads,
-// puts up to 16 waves on one CU's LDS; splitting the columns spreads them
-// over up to 8 CUs as long as every part keeps at least four waves.
+// How many workgroups share a head's value columns. A wide head as one
+// workgroup puts up to 16 waves on one CU's LDS (24 16-byte broadcast reads
+// per token and wave) and, at 128 registers a lane, spills; its columns are
+// shared out over up to 8 workgroups as long as every part keeps four waves.
+// The rule does not look at the batch, so a sequence takes the same path
+// whatever runs beside it.
 static int ls_splits(int mode, int S_, int H, int D, int DV) {
+  (void)S_;
+  (void)H;
   const int dkp = ls_pad(D);
   if (dkp == 0) return 1;
   const int P0 = dkp >= 64 ? 4 : (dkp >= 32 ? 2 : 1);
   if ((DV + (mode == LS_MLSTM ? 1 : 0)) * P0 > 1024) return 1;
-  const long wgs = (long)S_ * H;
   int cs = 1;
-  while (cs < 8 && wgs * cs * 2 <= 512 && DV % (cs * 2) == 0 &&
-         (DV / (cs * 2)) * P0 >= 256)
-    cs *= 2;
+  while (cs < 8 && DV % (cs * 2) == 0 && (DV / (cs * 2)) * P0 >= 256) cs *= 2;
   return cs;
 }
 

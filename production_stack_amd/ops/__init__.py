@@ -1020,9 +1020,9 @@ def linear_scan(mode: str, q, k, v, dec, gate, state, seq_rows, heads: int,
         return out
     _check_seq_rows(seq_rows)
     assert state.is_contiguous() and (aux is None or aux.is_contiguous())
-    # few (segment, head) pairs with wide heads: a head's value columns are
-    # shared out over several workgroups and the read-out norm runs as a
-    # second kernel over this fp32 scratch
+    # wide heads: a head's value columns are shared out over several
+    # workgroups and the read-out norm runs as a second kernel over this
+    # fp32 scratch
     raw = None
     if mode != "ssd" and _mx().mx_linear_scan_splits(
             SCAN_MODES[mode], seq_rows.shape[0], H, D, DV) > 1:
