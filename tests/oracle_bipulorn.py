@@ -9,8 +9,6 @@ groups, D key width, DV value width, N state size of the state-space mixer.
 
 from __future__ import annotations
 
-import math
-
 import torch
 
 F64 = torch.float64
