@@ -261,6 +261,13 @@ OTHER_STACKS = [
       (pair(2, 2, 8, 8, 5, 0.35, 4, 10.0, 1.0, 3, 10, 70, 1, 2, 2),
        moe(8, 2, 1, 2, 1.0, 8))],
      40, 29, 1e-5, 0.0, 2),
+    # heads wide enough for the scan kernel to share their value columns
+    # out over several workgroups (all three decay laws)
+    ([(gla(2, 64, 128, 4.0), None),
+      (mlstm(1, 64, 128, 8.0), moe(16, 4, 1, 2, 1.0, 16)),
+      (pair(2, 1, 16, 16, 12, 0.3, 8, 100.0, 2.0, 2, 128, 64, 1, 2, 3),
+       None)],
+     64, 37, 1e-5, 10.0, 4),
 ]
 
 
