@@ -56,7 +56,22 @@ class MixerSpec:
     `norm_groups` parts); "mlstm" has exponential input/forget gates capped
     at +-`gate_cap`, a running maximum and a normaliser.
     kind "pair": two mixers `left` and `right` read the same input; the
-    result is the mean of their separately normalised outputs.
+    result is the mean of their separately normalised outputs, or
+    (`combine` "weighted") left_scale * left + right_scale * right.
+    Attention options of the windowed kind: `window_pool` = P > 0 adds, for
+    every block of P consecutive positions that lies wholly before a
+    query's window, one key and value (the block's means as cached) to the
+    softmax; `qk_norm_all` RMS-normalises the whole query (and key)
+    projection at once, weights of that full size; `rot_layout` "half"
+    pairs entry i with entry i + rot_dims/2 instead of its neighbour;
+    `rot_scaling` = (factor, original length, fast turns, slow turns)
+    blends every frequency between itself and itself / factor by where its
+    number of turns over the original length falls, and scales cos/sin by
+    0.1 ln(factor) + 1.
+    kind "mingru": an element-wise gated recurrence over `vdim` channels
+    (heads = 1) whose gate and candidate read the current token only:
+    S <- (1 - z) S + z c, z = sigmoid(W_z h + b_z), c = u + 1/2 for
+    u = W_x h + b_x >= 0 and sigmoid(u) below; read-out S silu(W_g h).
     """
 
     kind: str
@@ -93,6 +108,13 @@ class MixerSpec:
     gate_cap: float = 0.0
     left: Optional["MixerSpec"] = None
     right: Optional["MixerSpec"] = None
+    window_pool: int = 0
+    qk_norm_all: bool = False
+    rot_layout: str = "interleaved"   # interleaved | half
+    rot_scaling: Optional[tuple] = None
+    combine: str = "norm_mean"        # norm_mean | weighted (pair)
+    left_scale: float = 1.0
+    right_scale: float = 1.0
 
 
 @dataclass
@@ -106,11 +128,14 @@ class MlpSpec:
     joins the scores for the choice only; `identity`: that many extra
     router outputs (after the experts) stand for experts that return their
     input; `route_scale` multiplies the final weights; `renorm_eps` is
-    added to the sum the chosen weights are divided by."""
+    added to the sum the chosen weights are divided by. `gated` False:
+    experts (and the shared expert) are down(act(up x)) without a gate
+    branch; `shared_gate` False: the shared expert joins unscaled. act
+    "relu2" is relu(z)^2."""
 
     kind: str
     ff: int
-    act: str = "silu"          # silu | gelu_tanh | clamped_swish
+    act: str = "silu"          # silu | gelu_tanh | clamped_swish | relu2
     limit: float = 0.0
     experts: int = 0
     top: int = 0
@@ -123,6 +148,8 @@ class MlpSpec:
     identity: int = 0
     route_scale: float = 1.0
     renorm_eps: float = 0.0
+    gated: bool = True
+    shared_gate: bool = True
 
 
 @dataclass
@@ -142,6 +169,12 @@ class LayerSpec:
     # joins the residual stream, and then scaled per channel (`layer_scale`)
     post_norm: bool = False
     layer_scale: bool = False
+    # "rms" or "layer" (mean removed, weight and bias)
+    norm: str = "rms"
+    # taps of the causal per-channel convolution over time that every
+    # sublayer's normed input h passes as h + conv(h) (0 = none); the last
+    # taps - 1 normed inputs of both sublayers are per-sequence state
+    input_conv: int = 0
 
 
 @dataclass
@@ -182,12 +215,17 @@ class ModelConfig:
     norm_groups: int = 1
     # logits become cap * tanh(logits / cap) (0 = off)
     logit_softcap: float = 0.0
+    # (start, stop, times): layers start .. stop-1 run `times` times in a
+    # row with the same weights, every pass with a cache and state of its
+    # own; each pass begins with x <- W_in [x; embedding output]
+    loop: Optional[tuple] = None
 
     @property
     def has_recurrent_state(self) -> bool:
         return bool(self.layer_specs) and any(
             ls.mixer.kind not in ("attention", "latent_attention")
-            or ls.token_shift for ls in self.layer_specs)
+            or ls.token_shift or ls.input_conv > 1
+            for ls in self.layer_specs)
 
     @property
     def q_size(self) -> int:

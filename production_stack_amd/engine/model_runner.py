@@ -171,6 +171,17 @@ class ModelRunner:
                         torch.zeros((num_blocks, heads, bs, dv), dtype=dt,
                                     device=self.device),
                     )
+                if kind == "kvpool":
+                    # paged keys/values plus one pooled key/value per
+                    # block of `pool` positions, in the page of the
+                    # block's first position
+                    _, heads, d, dv, pool = desc
+                    rows = (bs + pool - 1) // pool
+                    return tuple(
+                        torch.zeros((num_blocks, heads, r, w), dtype=dt,
+                                    device=self.device)
+                        for r, w in ((bs, d), (bs, dv), (rows, d),
+                                     (rows, dv)))
                 if kind == "paged":
                     # one paged tensor (keys that also hold the values)
                     _, heads, d = desc

@@ -99,13 +99,16 @@ def sparse_moe(x: torch.Tensor, weights: torch.Tensor, sel: torch.Tensor,
 class GatedMLP(nn.Module):
     """down(act(gate x) * up x); gate and up are one fused projection. The
     fused in-projection may be run by the caller together with other
-    consumers of the same input (see in_params / forward_from_proj)."""
+    consumers of the same input (see in_params / forward_from_proj).
+    gated False: down(act(up x)), `gate_up` then holds the up rows only."""
 
     def __init__(self, width: int, ff: int, act: str, limit: float,
-                 dtype: torch.dtype) -> None:
+                 dtype: torch.dtype, gated: bool = True) -> None:
         super().__init__()
-        self.ff, self.act, self.limit = ff, act, limit
-        self.gate_up = nn.Parameter(torch.empty(2 * ff, width, dtype=dtype))
+        self.ff, self.act, self.limit, self.gated = ff, act, limit, gated
+        self.in_rows = (2 if gated else 1) * ff
+        self.gate_up = nn.Parameter(
+            torch.empty(self.in_rows, width, dtype=dtype))
         self.down = nn.Parameter(torch.empty(width, ff, dtype=dtype))
 
     def in_params(self):
@@ -113,7 +116,10 @@ class GatedMLP(nn.Module):
 
     def inner(self, proj: torch.Tensor,
               out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """proj [T, 2*ff] = gate | up  ->  activation [T, ff]."""
+        """proj [T, 2*ff] = gate | up (or [T, ff] without a gate)  ->
+        activation [T, ff]."""
+        if not self.gated:
+            return ops.gated_act(proj, None, self.act, self.limit, out=out)
         return ops.gated_act(proj[:, :self.ff], proj[:, self.ff:], self.act,
                              self.limit, out=out)
 
@@ -139,16 +145,20 @@ class SparseMoE(nn.Module):
         self.correction = (
             nn.Parameter(torch.empty(E + spec.identity, dtype=torch.float32))
             if spec.correction else None)
+        # without a gate branch the tensor holds the up rows only
         self.experts_gate_up = nn.Parameter(
-            torch.empty(E, 2 * ff, width, dtype=dtype))
+            torch.empty(E, (2 if spec.gated else 1) * ff, width,
+                        dtype=dtype))
         self.experts_down = nn.Parameter(
             torch.empty(E, width, ff, dtype=dtype))
         self.shared = None
+        self.shared_gate = None
         if spec.shared_ff:
             self.shared = GatedMLP(width, spec.shared_ff, spec.act,
-                                   spec.shared_limit, dtype)
-            self.shared_gate = nn.Parameter(
-                torch.empty(1, width, dtype=dtype))
+                                   spec.shared_limit, dtype, spec.gated)
+            if spec.shared_gate:
+                self.shared_gate = nn.Parameter(
+                    torch.empty(1, width, dtype=dtype))
         self._fused_in = None
 
     def _apply(self, fn, *a, **kw):
@@ -176,6 +186,8 @@ class SparseMoE(nn.Module):
         gate."""
         if self.shared is None:
             return []
+        if self.shared_gate is None:
+            return [self.shared.gate_up]
         return [self.shared.gate_up, self.shared_gate]
 
     # decode-sized batches touch (nearly) every expert's weights anyway:
@@ -194,7 +206,8 @@ class SparseMoE(nn.Module):
         wm fp32 [T, router outputs]: the routing weights, zero where an
         output was not chosen. With the weight on the experts' outputs, the
         weighted sum, the identity outputs and the gated shared expert
-        (shared_y [T, W], shared_gate [T, 1] pre-sigmoid) are one kernel."""
+        (shared_y [T, W], shared_gate [T, 1] pre-sigmoid, None = joins
+        unscaled) are one kernel."""
         sp = self.spec
         T, E, ff = x.shape[0], sp.experts, sp.ff
         if sp.weight_on_input:
@@ -205,8 +218,11 @@ class SparseMoE(nn.Module):
         else:
             xe = x.unsqueeze(0).expand(E, T, x.shape[1])
         gu = torch.bmm(xe, self.experts_gate_up.transpose(1, 2))
-        gu2 = gu.view(E * T, 2 * ff)
-        act = ops.gated_act(gu2[:, :ff], gu2[:, ff:], sp.act, sp.limit)
+        gu2 = gu.view(E * T, gu.shape[2])
+        if sp.gated:
+            act = ops.gated_act(gu2[:, :ff], gu2[:, ff:], sp.act, sp.limit)
+        else:
+            act = ops.gated_act(gu2, None, sp.act, sp.limit, out=gu2)
         y = torch.bmm(act.view(E, T, ff), self.experts_down.transpose(1, 2))
         if not sp.weight_on_input:
             return ops.moe_combine(y, wm, x, E, shared_y, shared_gate)
@@ -214,7 +230,8 @@ class SparseMoE(nn.Module):
         if w_id is not None:
             y += x.float() * w_id
         if shared_y is not None:
-            y += shared_y.float() * torch.sigmoid(shared_gate.float())
+            y += (shared_y.float() * torch.sigmoid(shared_gate.float())
+                  if shared_gate is not None else shared_y.float())
         return y
 
     def _expert(self, e: int, xe: torch.Tensor) -> torch.Tensor:
@@ -222,15 +239,20 @@ class SparseMoE(nn.Module):
             return xe
         ff = self.spec.ff
         gu = gemm_policy.linear(xe, self.experts_gate_up[e])
-        act = ops.gated_act(gu[:, :ff], gu[:, ff:], self.spec.act,
-                            self.spec.limit)
+        if self.spec.gated:
+            act = ops.gated_act(gu[:, :ff], gu[:, ff:], self.spec.act,
+                                self.spec.limit)
+        else:
+            act = ops.gated_act(gu, None, self.spec.act, self.spec.limit,
+                                out=gu)
         return gemm_policy.linear(act, self.experts_down[e])
 
     def forward_from_proj(self, x: torch.Tensor,
                           proj: Optional[torch.Tensor],
                           dense: Optional[bool] = None) -> torch.Tensor:
         """x: layer input [T, width]; proj: the shared expert's fused
-        projection [T, 2*shared_ff + 1] (None without a shared expert).
+        projection [T, shared in-rows (+ 1 with a scalar gate)] (None
+        without a shared expert).
         dense=True insists on the all-experts path (no host read: what a
         captured decode step needs), None picks by batch size. Returns fp32
         [T, width]: several experts' outputs are summed in fp32."""
@@ -242,9 +264,10 @@ class SparseMoE(nn.Module):
         T = x.shape[0]
         y = gate = None
         if self.shared is not None:
-            sff = sp.shared_ff
-            y = self.shared.forward_from_proj(proj[:, :2 * sff])
-            gate = proj[:, 2 * sff:]
+            rows = self.shared.in_rows
+            y = self.shared.forward_from_proj(proj[:, :rows])
+            if self.shared_gate is not None:
+                gate = proj[:, rows:]
         if dense is None:
             dense = T <= self.DENSE_MAX_ROWS and T * sp.top >= sp.experts
         if dense:
@@ -253,7 +276,8 @@ class SparseMoE(nn.Module):
         sparse_moe(x, weights, sel, sp.experts + sp.identity, self._expert,
                    weight_on_input=sp.weight_on_input, out=out)
         if y is not None:
-            out += y.float() * torch.sigmoid(gate.float())
+            out += (y.float() * torch.sigmoid(gate.float())
+                    if gate is not None else y.float())
         return out
 
     def forward(self, x: torch.Tensor,

@@ -39,9 +39,14 @@ class TalkAttention(nn.Module):
     trailing-window visibility (with kept first keys), capped scores,
     denominator sink (fixed or learned), projection biases, per-head
     query/key norm, rotary position code on the leading entries of every
-    head (interleaved pairs, linear position scaling), value blending with
-    the stack's first value-mixing layer, a sigmoid output gate on the
-    concatenated heads; key and value widths may differ."""
+    head (interleaved or half-split pairs, linear position scaling or
+    blended frequencies), value blending with the stack's first
+    value-mixing layer, a sigmoid output gate on the concatenated heads;
+    key and value widths may differ. `window_pool`: blocks of positions
+    behind the window stay visible through one mean key/value each, kept in
+    a pooled cache that shares the pages of the key/value cache;
+    `qk_norm_all`: query and key are normalised over their whole
+    projections."""
 
     kind = "attention"
 
@@ -51,9 +56,8 @@ class TalkAttention(nn.Module):
         super().__init__()
         if spec.rope and spec.rot_dims <= 0:
             raise NotImplementedError(
-                "rotary attention here turns interleaved pairs of the "
-                "first rot_dims entries; the half-split layout is the "
-                "Llama attention path")
+                "rotary attention here turns pairs of the first rot_dims "
+                "entries of a head; give rot_dims")
         self.spec = spec
         self.max_pos = max_pos
         self._cos_sin = None
@@ -80,9 +84,18 @@ class TalkAttention(nn.Module):
             nn.Parameter(torch.empty(self.qkv.shape[0], dtype=dtype))
             if spec.bias else None)
         self.q_norm = self.k_norm = None
-        if spec.qk_norm:
+        if spec.qk_norm_all:
+            self.q_norm = nn.Parameter(
+                torch.empty(H * D, dtype=torch.float32))
+            self.k_norm = nn.Parameter(
+                torch.empty(G * D, dtype=torch.float32))
+        elif spec.qk_norm:
             self.q_norm = nn.Parameter(torch.empty(D, dtype=torch.float32))
             self.k_norm = nn.Parameter(torch.empty(D, dtype=torch.float32))
+        if spec.window_pool and not spec.window:
+            raise ValueError("pooled blocks need a window")
+        if spec.rot_layout not in ("interleaved", "half"):
+            raise ValueError(f"unknown rotary layout {spec.rot_layout!r}")
         self.sink_vals = (
             nn.Parameter(torch.empty(H, dtype=torch.float32))
             if spec.learned_sink else None)
@@ -103,7 +116,7 @@ class TalkAttention(nn.Module):
         cs = self._cos_sin
         if cs is None or cs.device != device:
             cs = ops.rope_table(self.max_pos, sp.rot_dims, sp.rot_base,
-                                device, sp.rot_factor)
+                                device, sp.rot_factor, sp.rot_scaling)
             self._cos_sin = cs
         return cs
 
@@ -126,18 +139,26 @@ class TalkAttention(nn.Module):
         return self.H * self.DV
 
     def cache_shape(self):
+        if self.spec.window_pool:
+            return ("kvpool", self.G, self.D, self.DV,
+                    self.spec.window_pool)
         return ("kv", self.G, self.D, self.DV)
 
     def forward_from_proj(self, proj: torch.Tensor, meta, cache,
                           out: Optional[torch.Tensor] = None,
                           shared: Optional[dict] = None) -> torch.Tensor:
         H, G, D, DV = self.H, self.G, self.D, self.DV
-        k_cache, v_cache = cache
+        sp = self.spec
+        pool = None
+        if sp.window_pool:
+            k_cache, v_cache, kp_cache, vp_cache = cache
+            pool = (kp_cache, vp_cache, sp.window_pool)
+        else:
+            k_cache, v_cache = cache
         q = proj[:, :H * D]
         k = proj[:, H * D:H * D + G * D]
         v = proj[:, H * D + G * D:self.qkv_rows]
-        sp = self.spec
-        if sp.qk_norm or sp.v_mix or sp.rope:
+        if sp.qk_norm or sp.qk_norm_all or sp.v_mix or sp.rope:
             # the first value-mixing layer of a step publishes its values;
             # later ones blend theirs with them before caching
             v_first = shared.get("v_first") if sp.v_mix else None
@@ -146,12 +167,19 @@ class TalkAttention(nn.Module):
                           meta.slot_mapping, H,
                           cos_sin=self.cos_sin(proj.device),
                           positions=meta.positions,
-                          rot_dims=sp.rot_dims if sp.rope else 0)
+                          rot_dims=sp.rot_dims if sp.rope else 0,
+                          norm_all=sp.qk_norm_all,
+                          half=sp.rot_layout == "half")
             if sp.v_mix and v_first is None:
                 shared["v_first"] = v
         else:
             ops.kv_append(k, v, k_cache, v_cache, meta.slot_mapping)
         T = proj.shape[0]
+        if pool is not None:
+            # blocks completed by this step's keys
+            ops.pool_append(k_cache, v_cache, kp_cache, vp_cache,
+                            meta.block_tables, meta.seq_rows,
+                            sp.window_pool, T)
         if out is None:
             out = torch.empty((T, H * DV), dtype=proj.dtype,
                               device=proj.device)
@@ -168,7 +196,7 @@ class TalkAttention(nn.Module):
                     chunk=sp.chunk, window=sp.window, sink=sp.sink,
                     talk=self.talk, out=out[a:b], variant=variant,
                     keep_first=sp.keep_first, softcap=sp.softcap,
-                    sink_vals=self.sink_vals)
+                    sink_vals=self.sink_vals, pool=pool)
         if sp.out_gate:
             ops.gated_act(proj[:, self.qkv_rows:], out, "sigmoid", out=out)
         return out
@@ -548,11 +576,44 @@ class StateSpaceDuality(_ScanMixer):
         return y
 
 
+class MinGRU(_ScanMixer):
+    """Minimal gated recurrent unit: an element-wise recurrence over
+    `vdim` channels whose gate and candidate read the current token only,
+    S <- (1 - z) S + z c with z = sigmoid(W_z h + b_z), u = W_x h + b_x,
+    c = u + 1/2 for u >= 0 and sigmoid(u) below; the read-out is
+    S silu(W_g h). Per sequence: S in fp32."""
+
+    kind = "mingru"
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float,
+                 dtype: torch.dtype) -> None:
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        C = spec.vdim or spec.dim
+        self.H, self.D, self.DV, self.C = 1, 1, C, C
+        # fused rows: gate | candidate | read-out gate
+        self.in_proj = nn.Parameter(torch.empty(3 * C, width, dtype=dtype))
+        self.z_bias = nn.Parameter(torch.empty(C, dtype=torch.float32))
+        self.x_bias = nn.Parameter(torch.empty(C, dtype=torch.float32))
+        self.out_weight = nn.Parameter(torch.empty(width, C, dtype=dtype))
+
+    def cache_shape(self):
+        return ("slots", (self.C,), torch.float32)
+
+    def forward_from_proj(self, proj, meta, cache, out=None):
+        C = self.C
+        return ops.mingru_scan(proj[:, :C], proj[:, C:2 * C],
+                               proj[:, 2 * C:3 * C], self.z_bias,
+                               self.x_bias, cache, meta.seq_rows, out=out)
+
+
 class MixerPair(nn.Module):
-    """Two mixers fed the same input: each half's projected
-    output is RMS-normalised over the model width with its own weight and
-    the result is their mean (fp32). Both input projections are one
-    GEMM."""
+    """Two mixers fed the same input. `combine` "norm_mean": each half's
+    projected output is RMS-normalised over the model width with its own
+    weight and the result is their mean (fp32); "weighted": the result is
+    left_scale * left + right_scale * right, which the caller's boundary
+    kernel adds to the stream in fp32 (forward_parts). Both input
+    projections are one GEMM."""
 
     kind = "pair"
 
@@ -562,10 +623,14 @@ class MixerPair(nn.Module):
         self.spec, self.eps = spec, eps
         self.left = build_mixer(width, spec.left, eps, dtype, max_pos)
         self.right = build_mixer(width, spec.right, eps, dtype, max_pos)
-        self.left_norm = nn.Parameter(torch.empty(width,
-                                                  dtype=torch.float32))
-        self.right_norm = nn.Parameter(torch.empty(width,
-                                                   dtype=torch.float32))
+        if spec.combine not in ("norm_mean", "weighted"):
+            raise ValueError(f"unknown pair combine {spec.combine!r}")
+        self.left_norm = self.right_norm = None
+        if spec.combine == "norm_mean":
+            self.left_norm = nn.Parameter(torch.empty(width,
+                                                      dtype=torch.float32))
+            self.right_norm = nn.Parameter(torch.empty(width,
+                                                       dtype=torch.float32))
         self._fused = None
 
     def cache_shape(self):
@@ -601,8 +666,8 @@ class MixerPair(nn.Module):
     def project(self, o: torch.Tensor) -> torch.Tensor:
         return o
 
-    def forward(self, h: torch.Tensor, meta, cache, shared: dict,
-                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward_parts(self, h: torch.Tensor, meta, cache, shared: dict):
+        """The halves' projected outputs (left, right)."""
         w, bias, n_left = self._fused or self.fuse()
         proj = (torch.addmm(bias, h, w.t()) if bias is not None
                 else gemm_policy.linear(h, w))
@@ -610,6 +675,14 @@ class MixerPair(nn.Module):
             proj[:, :n_left], meta, cache[0], None, shared))
         b = self.right.project(self.right.forward_from_proj(
             proj[:, n_left:], meta, cache[1]))
+        return a, b
+
+    def forward(self, h: torch.Tensor, meta, cache, shared: dict,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        a, b = self.forward_parts(h, meta, cache, shared)
+        if self.spec.combine == "weighted":
+            return (a.float() * self.spec.left_scale
+                    + b.float() * self.spec.right_scale)
         return ops.norm_sum32([a, b], [self.left_norm, self.right_norm],
                               0.5, self.eps)
 
@@ -624,6 +697,8 @@ def build_mixer(width: int, spec: MixerSpec, eps: float,
         return MatrixLSTM(width, spec, eps, dtype)
     if spec.kind == "ssd":
         return StateSpaceDuality(width, spec, eps, dtype)
+    if spec.kind == "mingru":
+        return MinGRU(width, spec, eps, dtype)
     if spec.kind == "pair":
         return MixerPair(width, spec, eps, dtype, max_pos)
     if spec.kind == "latent_attention":

@@ -45,11 +45,20 @@ def _bipulorn_cls():
     return BipulornForCausalLM
 
 
+def _dogidra_cls():
+    from production_stack_amd.engine.models.dogidra import (
+        DogidraForCausalLM,
+    )
+
+    return DogidraForCausalLM
+
+
 MODEL_CLASSES: Dict[str, Callable] = {
     "llama": _llama_cls,
     "nanurax": _nanurax_cls,
     "derusun": _derusun_cls,
     "bipulorn": _bipulorn_cls,
+    "dogidra": _dogidra_cls,
 }
 
 
@@ -72,14 +81,21 @@ def _bipulorn_config(path: str) -> ModelConfig:
     return bipulorn.config_from_dir(path)
 
 
+def _dogidra_config(path: str) -> ModelConfig:
+    from production_stack_amd.engine.models import dogidra
+
+    return dogidra.config_from_dir(path)
+
+
 CONFIG_READERS: Dict[str, Callable[[str], ModelConfig]] = {
     "Nanurax": _nanurax_config,
     "Derusun": _derusun_config,
     "Bipulorn": _bipulorn_config,
+    "Dogidra": _dogidra_config,
 }
 
 # families whose layers also run in float32 (the Llama path is bf16-only)
-FP32_FAMILIES = {"nanurax", "derusun", "bipulorn"}
+FP32_FAMILIES = {"nanurax", "derusun", "bipulorn", "dogidra"}
 
 
 def config_from_dir(path: str) -> ModelConfig:

@@ -416,7 +416,8 @@ def fp8_linear_rowwise(xq, sx, w_q, sw):
 # these run the kernels of `_mixops.so` (ops/native.py) for bf16 or float32
 # activations; on CPU tensors the references run.
 # ---------------------------------------------------------------------------
-ACT_KINDS = {"silu": 0, "gelu_tanh": 1, "clamped_swish": 2, "sigmoid": 3}
+ACT_KINDS = {"silu": 0, "gelu_tanh": 1, "clamped_swish": 2, "sigmoid": 3,
+             "relu2": 4}
 
 
 def _mx():
@@ -563,10 +564,11 @@ def depth_mix(hist: torch.Tensor, n: int, weights: torch.Tensor,
 def gated_act(gate: torch.Tensor, up: torch.Tensor, kind: str,
               limit: float = 0.0, out: torch.Tensor = None) -> torch.Tensor:
     """Gated-MLP inner activation on [T, F] views (row-strided allowed):
-    silu | gelu_tanh | clamped_swish | sigmoid (see reference.gated_act);
-    out may be up itself."""
+    silu | gelu_tanh | clamped_swish | sigmoid | relu2 (see
+    reference.gated_act); out may be up itself. up None: the plain
+    activation of `gate` (out may then be gate itself)."""
     T, F = gate.shape
-    assert up.shape == (T, F) and up.dtype == gate.dtype
+    assert up is None or (up.shape == (T, F) and up.dtype == gate.dtype)
     if out is None:
         out = torch.empty((T, F), dtype=gate.dtype, device=gate.device)
     assert out.shape == (T, F) and out.dtype == gate.dtype
@@ -575,7 +577,8 @@ def gated_act(gate: torch.Tensor, up: torch.Tensor, kind: str,
         return out
     _mx().mx_gated_act(
         _p(out), _rows(out, "out"), _p(gate), _rows(gate, "gate"), _p(up),
-        _rows(up, "up"), T, F, ACT_KINDS[kind], _f(limit),
+        _rows(up, "up") if up is not None else 0, T, F, ACT_KINDS[kind],
+        _f(limit),
         _mx_dtype(gate.dtype), _stream())
     return out
 
@@ -610,7 +613,7 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
                    out: torch.Tensor = None, variant: int = 0,
                    splits: int = 0, keep_first: int = 0,
                    softcap: float = 0.0, sink_vals: torch.Tensor = None,
-                   vdim: int = 0) -> torch.Tensor:
+                   vdim: int = 0, pool=None) -> torch.Tensor:
     """Paged attention of a ragged batch. q [T, H*D] (row-strided view
     allowed); token_seq/token_pos int32 [T] give each token's block-table
     row and position; talk: optional fp32 [H, H] score mix; chunk/window:
@@ -619,7 +622,10 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
     tanh(score / cap); sink: a value-less key joins the softmax
     denominator with score 0, or sink_vals[h] (fp32 [H]) when given; vdim:
     the values are the first vdim entries of v_cache's rows (v_cache may be
-    k_cache itself: keys that carry their values).
+    k_cache itself: keys that carry their values). pool = (kp_cache,
+    vp_cache, P): with a window, every block of P positions that lies
+    wholly before a query's window adds its pooled key and value (as
+    pool_append stores them) to the same softmax.
     variant 0 picks the kernel for prompt portions (tiled thread-per-
     (head, query) where the shape fits), 3 for single tokens (split-key),
     both falling back to the plain one-workgroup-per-token kernel; 1 / 2 /
@@ -642,6 +648,16 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
     if sink_vals is not None:
         assert sink and sink_vals.dtype == torch.float32
         assert sink_vals.shape == (H,)
+    kp = vp = None
+    P = PR = 0
+    if pool is not None and window > 0:
+        kp, vp, P = pool
+        PR = (BS + P - 1) // P
+        assert P >= 1 and chunk == 0 and keep_first == 0 and vdim == 0
+        assert kp.shape == (NB, G, PR, D) and vp.shape == (NB, G, PR, DV)
+        assert kp.dtype == k_cache.dtype and vp.dtype == v_cache.dtype
+    else:
+        pool = None
     if out is None:
         out = torch.empty((T, H * DV), dtype=q.dtype, device=q.device)
     assert out.shape == (T, H * DV) and out.dtype == q.dtype
@@ -649,7 +665,7 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
         o = reference.talk_attention(
             q.reshape(T, H, D), k_cache, v_cache, block_tables, token_seq,
             token_pos, scale, chunk, window, sink, talk, keep_first,
-            softcap, sink_vals, DV)
+            softcap, sink_vals, DV, pool)
         out.copy_(o.reshape(T, H * DV))
         return out
     assert q.dtype == k_cache.dtype == v_cache.dtype
@@ -657,6 +673,8 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
     assert block_tables.is_contiguous()
     if talk is not None:
         assert talk.is_contiguous()
+    if pool is not None:
+        assert kp.is_contiguous() and vp.is_contiguous()
     # single tokens: when the batch is too small to fill the chip with one
     # workgroup per token, each token's keys are shared out over several
     # workgroups whose partial softmax records are merged afterwards
@@ -683,7 +701,7 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
             int(window), int(bool(sink)), int(keep_first), _f(softcap),
             _p(sink_vals), int(VR),
             int(v_cache.data_ptr() == k_cache.data_ptr()), int(splits),
-            _p(scratch), mode, _stream())
+            _p(scratch), mode, _p(kp), _p(vp), int(P), _stream())
         if rc == 0:
             return out
     if variant in (5, 6):
@@ -695,7 +713,8 @@ def talk_attention(q: torch.Tensor, k_cache: torch.Tensor,
         _p(token_seq), _p(token_pos), _p(talk), T, H, G, D, DV, BS,
         _f(scale), int(chunk), int(window), int(bool(sink)),
         _mx_dtype(q.dtype), int(variant), int(splits), _p(scratch),
-        int(keep_first), _f(softcap), _p(sink_vals), int(VR), _stream())
+        int(keep_first), _f(softcap), _p(sink_vals), int(VR), _p(kp),
+        _p(vp), int(P), _stream())
     if rc != 0:
         raise RuntimeError(
             f"talk_attention: heads x dim {H}x{D}/{DV} exceeds the kernel's "
@@ -707,7 +726,8 @@ def attn_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
               q_w, k_w, eps: float, vmix, v_first, k_cache: torch.Tensor,
               v_cache: torch.Tensor, slot_mapping: torch.Tensor,
               heads: int, cos_sin: torch.Tensor = None,
-              positions: torch.Tensor = None, rot_dims: int = 0) -> None:
+              positions: torch.Tensor = None, rot_dims: int = 0,
+              norm_all: bool = False, half: bool = False) -> None:
     """Per-head query/key RMSNorm (weights q_w / k_w fp32 [D], None = no
     norm; q is rewritten in place), value blend (1 - vmix) v + vmix v_first
     when v_first [T, G*DV] is given (vmix a 0-dim fp32 tensor; v is
@@ -715,7 +735,10 @@ def attn_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     query and key head (cos_sin fp32 [positions, rot_dims/2, 2] as
     rope_table builds it, positions int32 [T]; interleaved pairs; q is
     rewritten in place), and append of the keys and values to the paged
-    caches [NB, G, BS, D|DV]. q/k/v are row-strided views."""
+    caches [NB, G, BS, D|DV]. q/k/v are row-strided views. norm_all: one
+    root mean square over the whole query (key) projection and weights
+    q_w fp32 [H*D] / k_w fp32 [G*D]; half: the rotary pairs are (i, i +
+    rot_dims/2) instead of (2i, 2i+1)."""
     NB, G, BS, D = k_cache.shape
     DV = v_cache.shape[3]
     T = q.shape[0]
@@ -734,13 +757,14 @@ def attn_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     if not q.is_cuda:
         reference.attn_prep(q, k, v, q_w, k_w, eps, vmix, v_first, k_cache,
                             v_cache, slot_mapping, H, cos_sin, positions,
-                            rot_dims)
+                            rot_dims, norm_all, half)
         return
     assert q.dtype == k.dtype == v.dtype == k_cache.dtype == v_cache.dtype
     assert k_cache.is_contiguous() and v_cache.is_contiguous()
-    for w in (q_w, k_w):
+    for w, n in ((q_w, H), (k_w, G)):
         if w is not None:
-            assert w.dtype == torch.float32 and w.numel() == D
+            assert w.dtype == torch.float32
+            assert w.numel() == (n * D if norm_all else D)
     _mx().mx_attn_prep(
         _p(q), _rows(q, "q"), _p(k), _rows(k, "k"), _p(v), _rows(v, "v"),
         _p(q_w), _p(k_w), _f(eps), _p(vmix if v_first is not None else None),
@@ -748,14 +772,142 @@ def attn_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         _p(k_cache), _p(v_cache), _p(slot_mapping), T, H, G, D, DV, BS,
         _p(cos_sin), int(cos_sin.shape[0]) if cos_sin is not None else 0,
         int(rot_dims) if cos_sin is not None else 0, _p(positions),
-        _mx_dtype(q.dtype), _stream())
+        int(bool(norm_all)), int(bool(half)), _mx_dtype(q.dtype), _stream())
 
 
 def rope_table(max_pos: int, dims: int, base: float,
-               device=None, factor: float = 1.0) -> torch.Tensor:
+               device=None, factor: float = 1.0,
+               scaling=None) -> torch.Tensor:
     """fp32 [max_pos, dims/2, 2] (cos, sin) of position * base^(-2i/dims)
-    / factor, correctly rounded (angles formed in float64 on the host)."""
-    return reference.rope_table(max_pos, dims, base, device, factor)
+    / factor, correctly rounded (angles formed in float64 on the host);
+    scaling = (factor, original, fast, slow) blends the frequencies and
+    scales the magnitude (see reference.scaled_frequencies)."""
+    return reference.rope_table(max_pos, dims, base, device, factor,
+                                scaling)
+
+
+def pool_append(k_cache: torch.Tensor, v_cache: torch.Tensor,
+                kp_cache: torch.Tensor, vp_cache: torch.Tensor,
+                block_tables: torch.Tensor, seq_rows: torch.Tensor,
+                pool: int, num_tokens: int) -> None:
+    """Stores the mean key and value of every block of `pool` consecutive
+    positions that this step completed (see reference.pool_append):
+    caches [NB, G, BS, D|DV] -> pooled caches [NB, G, ceil(BS/pool),
+    D|DV]. Runs after the step's keys and values were appended;
+    num_tokens is the step's row count (bounds a segment's blocks)."""
+    NB, G, BS, D = k_cache.shape
+    DV = v_cache.shape[3]
+    PR = (BS + pool - 1) // pool
+    assert pool >= 1 and kp_cache.shape == (NB, G, PR, D)
+    assert vp_cache.shape == (NB, G, PR, DV)
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2
+    assert block_tables.shape[0] == seq_rows.shape[0]
+    if not k_cache.is_cuda:
+        reference.pool_append(k_cache, v_cache, kp_cache, vp_cache,
+                              block_tables, seq_rows, pool)
+        return
+    _check_seq_rows(seq_rows)
+    assert k_cache.dtype == v_cache.dtype == kp_cache.dtype == vp_cache.dtype
+    for t in (k_cache, v_cache, kp_cache, vp_cache, block_tables):
+        assert t.is_contiguous()
+    S = seq_rows.shape[0]
+    # a segment of n rows completes at most n // pool + 1 blocks
+    longest = num_tokens - (S - 1)
+    _mx().mx_pool_append(
+        _p(k_cache), _p(v_cache), _p(kp_cache), _p(vp_cache),
+        _p(block_tables), block_tables.shape[1], _p(seq_rows), S,
+        longest // pool + 1, G, D, DV, BS, int(pool),
+        _mx_dtype(k_cache.dtype), _stream())
+
+
+def add_layer_norm_conv32(x32: torch.Tensor, deltas, scales,
+                          w32: torch.Tensor, b32: torch.Tensor, eps: float,
+                          conv_w: torch.Tensor, state: torch.Tensor,
+                          seq_rows: torch.Tensor,
+                          out_dtype: torch.dtype) -> torch.Tensor:
+    """Sublayer boundary with a layer norm and an input convolution (see
+    reference.add_layer_norm_conv32): x32 fp32 [T, W] += sum scales[i] *
+    deltas[i] in place (up to two deltas [T, W] of one dtype, row-strided
+    views allowed), y = layernorm(x32) * w32 + b32, returns y + conv(y) in
+    out_dtype, the causal convolution (conv_w fp32 [W, K]) running along
+    the segments of seq_rows with state fp32 [slots, K-1, W] (a segment's
+    previous K - 1 rows of y), which is updated. conv_w None: returns y."""
+    T, W = x32.shape
+    assert x32.dtype == torch.float32 and x32.is_contiguous()
+    deltas, scales = list(deltas), [float(v) for v in scales]
+    assert len(deltas) <= 2 and len(scales) == len(deltas)
+    for d in deltas:
+        assert d.shape == (T, W) and d.dtype == deltas[0].dtype
+    for w in (w32, b32):
+        assert w.dtype == torch.float32 and w.numel() == W
+    K = 0
+    if conv_w is not None:
+        K = conv_w.shape[1]
+        assert conv_w.dtype == torch.float32 and conv_w.shape == (W, K)
+        assert K >= 1 and state.dtype == torch.float32
+        assert state.shape[1:] == (K - 1, W)
+    if not x32.is_cuda:
+        return reference.add_layer_norm_conv32(
+            x32, deltas, scales, w32, b32, eps, conv_w, state, seq_rows,
+            out_dtype)
+    h = torch.empty((T, W), dtype=out_dtype, device=x32.device)
+    stats = None
+    if conv_w is not None:
+        _check_seq_rows(seq_rows)
+        assert conv_w.is_contiguous() and state.is_contiguous()
+        stats = torch.empty((T, 2), dtype=torch.float32, device=x32.device)
+    d0 = deltas[0] if deltas else None
+    d1 = deltas[1] if len(deltas) > 1 else None
+    _mx().mx_add_layer_norm32(
+        _p(h if conv_w is None else None), _p(x32), _p(d0),
+        _rows(d0, "delta") if d0 is not None else 0,
+        _f(scales[0] if deltas else 0.0), _p(d1),
+        _rows(d1, "delta") if d1 is not None else 0,
+        _f(scales[1] if d1 is not None else 0.0), _p(w32), _p(b32), _f(eps),
+        _p(stats), T, W,
+        _mx_dtype(d0.dtype) if d0 is not None else 0, _mx_dtype(out_dtype),
+        _stream())
+    if conv_w is not None:
+        S = seq_rows.shape[0]
+        rc = _mx().mx_norm_conv32(
+            _p(h), _p(x32), _p(stats), _p(w32), _p(b32), _p(conv_w),
+            _p(state), _p(seq_rows), S, W, K, T, _mx_dtype(out_dtype),
+            _stream())
+        if rc != 0:
+            raise RuntimeError(
+                f"add_layer_norm_conv32: {K} taps are not built (1-8)")
+    return h
+
+
+def mingru_scan(z: torch.Tensor, u: torch.Tensor, g: torch.Tensor,
+                zb: torch.Tensor, ub: torch.Tensor, state: torch.Tensor,
+                seq_rows: torch.Tensor,
+                out: torch.Tensor = None) -> torch.Tensor:
+    """Element-wise gated recurrence S <- (1 - a) S + a c over a ragged
+    batch with read-out S * silu(g) (see reference.mingru_scan). z / u / g
+    [T, C] row-strided views of one dtype; zb / ub fp32 [C]; state fp32
+    [slots, C], updated in place. Returns [T, C] of the inputs' dtype."""
+    T, C = z.shape
+    assert u.shape == (T, C) and g.shape == (T, C)
+    assert u.dtype == z.dtype and g.dtype == z.dtype
+    assert state.dtype == torch.float32 and state.shape[1:] == (C,)
+    for b in (zb, ub):
+        assert b.dtype == torch.float32 and b.numel() == C
+    if out is None:
+        out = torch.empty((T, C), dtype=z.dtype, device=z.device)
+    assert out.shape == (T, C) and out.dtype == z.dtype
+    if not z.is_cuda:
+        out.copy_(reference.mingru_scan(z, u, g, zb, ub, state, seq_rows,
+                                        z.dtype))
+        return out
+    _check_seq_rows(seq_rows)
+    assert state.is_contiguous()
+    _mx().mx_mingru_scan(
+        _p(out), _rows(out, "out"), _p(z), _rows(z, "z"), _p(u),
+        _rows(u, "u"), _p(g), _rows(g, "g"), _p(zb), _p(ub), _p(state),
+        _p(seq_rows), seq_rows.shape[0], C, T, _mx_dtype(z.dtype),
+        _stream())
+    return out
 
 
 def latent_prep(q_lat: torch.Tensor, q: torch.Tensor, dkv: torch.Tensor,
@@ -1050,7 +1202,7 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, top: int,
     """Router of a routed feed-forward in one kernel (see
     reference.moe_route): fp32 logits of x [T, W] against router_w
     [n_out, W] (both of the serving dtype), softmax or sigmoid scores, the
-    `top` best by score + correction (fp32 [n_out], softmax only), weights
+    `top` best by score + correction (fp32 [n_out]), weights
     = chosen scores / (sum + renorm_eps) when renormalize, times scale.
     Returns (weights fp32 [T, top], indices int64 [T, top], dense fp32
     [T, n_out] with the weights at the chosen outputs and zeros
@@ -1060,7 +1212,7 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, top: int,
     assert router_w.shape == (n_out, W) and router_w.dtype == x.dtype
     assert score in ("softmax", "sigmoid") and 1 <= top <= n_out
     if correction is not None:
-        assert score == "softmax" and correction.dtype == torch.float32
+        assert correction.dtype == torch.float32
         assert correction.shape == (n_out,)
     if not x.is_cuda:
         return reference.moe_route(x, router_w, top, score, renormalize,
@@ -1086,16 +1238,18 @@ def moe_combine(y: torch.Tensor, dense: torch.Tensor, x: torch.Tensor,
     every expert's output for every row, dense fp32 [T, n_out] the routing
     weights (zero = not chosen; outputs from `experts` on are identity
     outputs that return the input x [T, W]); the shared expert's output
-    shared_y [T, W] joins times sigmoid(shared_gate [T, 1]). Returns fp32
-    [T, W]."""
+    shared_y [T, W] joins times sigmoid(shared_gate [T, 1]) (unscaled when
+    shared_gate is None). Returns fp32 [T, W]."""
     E, T, W = y.shape
     n_out = dense.shape[1]
     assert E == experts and n_out >= E and dense.shape == (T, n_out)
     assert dense.dtype == torch.float32 and x.shape == (T, W)
     assert x.dtype == y.dtype
     if shared_y is not None:
-        assert shared_y.shape == (T, W) and shared_gate.shape == (T, 1)
-        assert shared_y.dtype == y.dtype and shared_gate.dtype == y.dtype
+        assert shared_y.shape == (T, W) and shared_y.dtype == y.dtype
+        if shared_gate is not None:
+            assert shared_gate.shape == (T, 1)
+            assert shared_gate.dtype == y.dtype
     if not y.is_cuda:
         return reference.moe_combine(y, dense, x, experts, shared_y,
                                      shared_gate)

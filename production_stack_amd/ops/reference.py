@@ -12,6 +12,8 @@ They intentionally mirror the kernel semantics exactly (paged cache layout
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 
@@ -264,17 +266,21 @@ def gated_act(gate, up, kind: str, limit: float, out_dtype):
     """Gated-MLP inner activation, fp32 math, one rounding at the end.
     silu: silu(g)*u; gelu_tanh: gelu_tanh(g)*u; clamped_swish:
     g' = min(g, limit), u' = clamp(u, +-limit), g' sigmoid(1.702 g') (u'+1);
-    sigmoid: sigmoid(g)*u (an output gate).
+    sigmoid: sigmoid(g)*u (an output gate); relu2: relu(g)^2 * u. up None:
+    the plain activation (u = 1).
     """
     g = gate.float()
-    u = up.float()
-    if kind == "silu":
+    u = up.float() if up is not None else 1.0
+    if kind == "relu2":
+        y = torch.relu(g).pow(2) * u
+    elif kind == "silu":
         y = torch.nn.functional.silu(g) * u
     elif kind == "gelu_tanh":
         y = torch.nn.functional.gelu(g, approximate="tanh") * u
     elif kind == "clamped_swish":
         g = torch.clamp(g, max=limit)
-        u = torch.clamp(u, min=-limit, max=limit)
+        u = (torch.clamp(u, min=-limit, max=limit) if up is not None
+             else 0.0)
         y = g * torch.sigmoid(1.702 * g) * (u + 1.0)
     elif kind == "sigmoid":
         y = torch.sigmoid(g) * u
@@ -296,13 +302,16 @@ def kv_append(k, v, k_cache, v_cache, slot_mapping) -> None:
 def talk_attention(q, k_cache, v_cache, block_tables, token_seq, token_pos,
                    scale: float, chunk: int, window: int, sink: bool,
                    talk, keep_first: int = 0, softcap: float = 0.0,
-                   sink_vals=None, vdim: int = 0):
+                   sink_vals=None, vdim: int = 0, pool=None):
     """Paged attention with optional head-mixed scores, aligned-chunk or
     trailing-window visibility (the first keep_first keys stay visible
     behind the window), capped scores and a denominator sink (score 0, or
     sink_vals[h]). q [T, H, D]; the values are the first vdim entries of
     v_cache rows (all of them when 0; v_cache may be k_cache). Returns
-    [T, H, DV] in q's dtype; all score math in fp32."""
+    [T, H, DV] in q's dtype; all score math in fp32. pool = (kp_cache,
+    vp_cache, P): with a window, every block of P positions whose last
+    position is at or before pos - window adds its pooled key/value (see
+    pool_append) to the same softmax."""
     T, H, D = q.shape
     G, bs = v_cache.shape[1], v_cache.shape[2]
     DV = vdim or v_cache.shape[3]
@@ -324,6 +333,14 @@ def talk_attention(q, k_cache, v_cache, block_tables, token_seq, token_pos,
         off = idx % bs
         kk = k_cache[blk, :, off].float()          # [n, G, D]
         vv = v_cache[blk, :, off][..., :DV].float()  # [n, G, DV]
+        if pool is not None and window > 0:
+            kp, vp, P = pool
+            nb = max(0, (pos - window + 1) // P)
+            if nb:
+                first = torch.arange(nb) * P
+                pb, po = table[first // bs], (first % bs) // P
+                kk = torch.cat([kp[pb, :, po].float(), kk])
+                vv = torch.cat([vp[pb, :, po][..., :DV].float(), vv])
         kk = kk.repeat_interleave(rep, dim=1)      # [n, H, D]
         vv = vv.repeat_interleave(rep, dim=1)
         s = torch.einsum("hd,nhd->hn", q[t].float(), kk) * scale
@@ -346,7 +363,8 @@ def talk_attention(q, k_cache, v_cache, block_tables, token_seq, token_pos,
 
 def attn_prep(q, k, v, q_w, k_w, eps: float, vmix, v_first, k_cache,
               v_cache, slot_mapping, heads: int, cos_sin=None,
-              positions=None, rot_dims: int = 0):
+              positions=None, rot_dims: int = 0, norm_all: bool = False,
+              half: bool = False):
     """Query/key head norm, value blend and cache append of one attention
     layer. q [T, H*D] is normalised in place per head (x / rms(x) * q_w,
     fp32 math); k [T, G*D] likewise with k_w and appended; v [T, G*DV]
@@ -354,7 +372,9 @@ def attn_prep(q, k, v, q_w, k_w, eps: float, vmix, v_first, k_cache,
     0-dim fp32 tensor), is written back, and appended. q_w / k_w None:
     no norm. With cos_sin (fp32 [positions, rot_dims/2, 2]) the first
     rot_dims entries of every query and key head turn by the row of the
-    token's position (interleaved pairs), after the norm."""
+    token's position (interleaved pairs, or with `half` entry i paired
+    with entry i + rot_dims/2), after the norm. norm_all: q_w [H*D] / k_w
+    [G*D] and one root mean square over the whole projection."""
     T = q.shape[0]
     G, bs, D = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     DV = v_cache.shape[3]
@@ -362,16 +382,17 @@ def attn_prep(q, k, v, q_w, k_w, eps: float, vmix, v_first, k_cache,
     if q_w is not None or cs is not None:
         qf = q.float().view(T, heads, D)
         if q_w is not None:
-            qf = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True)
-                                  + eps) * q_w
+            qf = _unit_heads(qf, eps, norm_all) * q_w.view(
+                (1, heads, D) if norm_all else (1, 1, D))
         if cs is not None:
-            qf = _rotate(qf, cs, rot_dims)
+            qf = _rotate(qf, cs, rot_dims, half)
         q.copy_(qf.reshape(T, heads * D).to(q.dtype))
     kf = k.float().view(T, G, D)
     if k_w is not None:
-        kf = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) * k_w
+        kf = _unit_heads(kf, eps, norm_all) * k_w.view(
+            (1, G, D) if norm_all else (1, 1, D))
     if cs is not None:
-        kf = _rotate(kf, cs, rot_dims)
+        kf = _rotate(kf, cs, rot_dims, half)
     vf = v.float()
     if v_first is not None:
         lam = vmix.float()
@@ -380,28 +401,149 @@ def attn_prep(q, k, v, q_w, k_w, eps: float, vmix, v_first, k_cache,
     kv_append(kf, vf.view(T, G, DV), k_cache, v_cache, slot_mapping)
 
 
-def rope_table(max_pos: int, dims: int, base: float, device=None,
-               factor: float = 1.0):
-    """fp32 [max_pos, dims/2, 2] = (cos, sin) of position * base^(-2i/dims)
-    / factor (linear position scaling). The angles are formed in float64 on
-    the host, so an entry is the correctly rounded fp32 value."""
-    i = torch.arange(0, dims, 2, dtype=torch.float64)
+def _unit_heads(x, eps: float, whole: bool):
+    """x fp32 [T, heads, D] over its root mean square per head, or over all
+    heads at once."""
+    ms = (x.pow(2).mean((-2, -1), keepdim=True) if whole
+          else x.pow(2).mean(-1, keepdim=True))
+    return x * torch.rsqrt(ms + eps)
+
+
+def scaled_frequencies(dims: int, base: float, scaling=None):
+    """float64 [dims/2] angular frequencies base^(-2i/dims) and the common
+    magnitude of cos/sin. scaling = (factor, original, fast, slow): with
+    d(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(
+    d(fast)), 0), hi = min(ceil(d(slow)), dims - 1) and ramp_i =
+    clamp((i - lo) / max(hi - lo, 0.001), 0, 1), frequency i becomes
+    f_i / factor * ramp_i + f_i (1 - ramp_i); the magnitude is
+    0.1 ln(factor) + 1."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
     f = torch.pow(torch.tensor(float(base), dtype=torch.float64),
-                  -i / dims) / float(factor)
+                  -2.0 * i / dims)
+    if not scaling:
+        return f, 1.0
+    factor, original, fast, slow = (float(v) for v in scaling)
+
+    def d_of(turns):
+        return dims * math.log(original / (2.0 * math.pi * turns)) / (
+            2.0 * math.log(base))
+
+    lo = max(math.floor(d_of(fast)), 0)
+    hi = min(math.ceil(d_of(slow)), dims - 1)
+    ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    return f / factor * ramp + f * (1.0 - ramp), 0.1 * math.log(factor) + 1.0
+
+
+def rope_table(max_pos: int, dims: int, base: float, device=None,
+               factor: float = 1.0, scaling=None):
+    """fp32 [max_pos, dims/2, 2] = (cos, sin) of position * base^(-2i/dims)
+    / factor (linear position scaling); with `scaling` the frequencies and
+    the magnitude of scaled_frequencies. The angles are formed in float64
+    on the host, so an entry is the correctly rounded fp32 value."""
+    f, mag = scaled_frequencies(dims, base, scaling)
+    f = f / float(factor)
     a = torch.arange(max_pos, dtype=torch.float64)[:, None] * f
-    t = torch.stack([torch.cos(a), torch.sin(a)], dim=-1).float()
+    t = (torch.stack([torch.cos(a), torch.sin(a)], dim=-1) * mag).float()
     return t.to(device).contiguous() if device is not None else t.contiguous()
 
 
-def _rotate(x, cs, dims: int):
-    """x fp32 [..., n]; cs [..., dims/2, 2] broadcastable; interleaved
-    pairs (2i, 2i+1) of the first dims entries turn."""
+def _rotate(x, cs, dims: int, half: bool = False):
+    """x fp32 [..., n]; cs [..., dims/2, 2] broadcastable; pairs of the
+    first dims entries turn: interleaved (2i, 2i+1), or (i, i + dims/2)
+    with `half`."""
     x = x.clone()
-    u, w = x[..., 0:dims:2].clone(), x[..., 1:dims:2].clone()
+    if half:
+        a, b = slice(0, dims // 2), slice(dims // 2, dims)
+    else:
+        a, b = slice(0, dims, 2), slice(1, dims, 2)
+    u, w = x[..., a].clone(), x[..., b].clone()
     c, s = cs[..., 0], cs[..., 1]
-    x[..., 0:dims:2] = u * c - w * s
-    x[..., 1:dims:2] = w * c + u * s
+    x[..., a] = u * c - w * s
+    x[..., b] = w * c + u * s
     return x
+
+
+def pool_append(k_cache, v_cache, kp_cache, vp_cache, block_tables,
+                seq_rows, pool: int) -> None:
+    """Pooled keys/values of the blocks of `pool` consecutive positions
+    that this step completes. Block b holds positions b*pool .. b*pool +
+    pool - 1; once its last position is cached, the fp32 means of its keys
+    and of its values, as the caches [NB, G, BS, D|DV] hold them, are
+    stored (rounded to the cache dtype) in kp_cache / vp_cache [NB, G,
+    ceil(BS / pool), D|DV]: in the page of the block's first position, at
+    row (first position mod BS) div pool. seq_rows row i = (first batch
+    row, rows, first position, slot) and block_tables row i belong to
+    segment i."""
+    bs = k_cache.shape[2]
+    for i, (_, n, p0, _) in enumerate(seq_rows.tolist()):
+        table = block_tables[i].long()
+        # blocks whose last position lies in [p0, p0 + n)
+        for b in range(p0 // pool, (p0 + n) // pool):
+            idx = torch.arange(b * pool, (b + 1) * pool)
+            blk, off = table[idx // bs], idx % bs
+            page, row = table[(b * pool) // bs], ((b * pool) % bs) // pool
+            kp_cache[page, :, row] = k_cache[blk, :, off].float().mean(0).to(
+                kp_cache.dtype)
+            vp_cache[page, :, row] = v_cache[blk, :, off].float().mean(0).to(
+                vp_cache.dtype)
+
+
+def add_layer_norm_conv32(x32, deltas, scales, w32, b32, eps: float,
+                          conv_w, state, seq_rows, out_dtype):
+    """Sublayer boundary of a stack with layer norms and input
+    convolutions: x32 += sum_i scales[i] * deltas[i] (fp32, in place), y =
+    (x32 - mean) / sqrt(var + eps) * w32 + b32 per row, and the returned
+    h = y + conv(y) in out_dtype, conv(y)_t = sum_j conv_w[:, j] *
+    y_(t - K + 1 + j) along each segment of seq_rows with the segment's
+    previous K - 1 rows of y taken from state fp32 [slots, K-1, W] (zeros
+    for a segment that starts at position 0); state receives the last K - 1
+    rows. conv_w None: h = y."""
+    if deltas:
+        acc = None
+        for d, sc in zip(deltas, scales):
+            term = d.float() * sc
+            acc = term if acc is None else acc + term
+        x32.add_(acc)
+    mu = x32.mean(-1, keepdim=True)
+    var = (x32 - mu).pow(2).mean(-1, keepdim=True)
+    y = (x32 - mu) * torch.rsqrt(var + eps) * w32 + b32
+    if conv_w is None:
+        return y.to(out_dtype)
+    T, W = y.shape
+    K = conv_w.shape[1]
+    h = torch.empty_like(y)
+    for t0, n, p0, slot in seq_rows.tolist():
+        past = state[slot] if p0 > 0 else torch.zeros(K - 1, W)
+        ext = torch.cat([past, y[t0:t0 + n]], dim=0)
+        acc = y[t0:t0 + n].clone()
+        for j in range(K):
+            acc += ext[j:j + n] * conv_w[:, j]
+        h[t0:t0 + n] = acc
+        if K > 1:
+            state[slot] = ext[n:]
+    return h.to(out_dtype)
+
+
+def mingru_scan(z, u, g, zb, ub, state, seq_rows, out_dtype):
+    """Element-wise gated recurrence over a ragged batch. z / u / g [T, C]
+    (gate, candidate and read-out projections), zb / ub fp32 [C] their
+    biases; state fp32 [slots, C], updated in place, zeros for a segment
+    that starts at position 0. Per token a = sigmoid(z + zb), c = u + ub +
+    1/2 where u + ub >= 0 and sigmoid(u + ub) below, S <- (1 - a) S + a c;
+    returns S * silu(g) in out_dtype. All arithmetic fp32."""
+    a = torch.sigmoid(z.float() + zb)
+    uu = u.float() + ub
+    c = torch.where(uu >= 0, uu + 0.5, torch.sigmoid(uu))
+    T, C = a.shape
+    y = torch.empty(T, C, dtype=torch.float32)
+    for t0, n, p0, slot in seq_rows.tolist():
+        S = state[slot].clone() if p0 > 0 else torch.zeros(C)
+        for t in range(t0, t0 + n):
+            S = (1.0 - a[t]) * S + a[t] * c[t]
+            y[t] = S
+        state[slot] = S
+    gf = g.float()
+    return (y * gf * torch.sigmoid(gf)).to(out_dtype)
 
 
 def latent_prep(q_lat, q, dkv, norm_w, eps: float, cos_sin, positions,
@@ -637,7 +779,8 @@ def moe_route(x, router_w, top: int, score: str, renormalize: bool,
               correction, scale: float, renorm_eps: float):
     """Router of a routed feed-forward: fp32 logits, softmax | sigmoid
     scores, the `top` outputs with the largest score + correction (sigmoid
-    scores are ranked by their logits), weights = chosen scores, divided by
+    scores without a correction are ranked by their logits), weights =
+    chosen scores, divided by
     (their sum + renorm_eps) when renormalize, times scale. Returns
     (weights [T, top], indices [T, top], dense [T, n_out])."""
     logits = torch.nn.functional.linear(x.float(), router_w.float())
@@ -646,7 +789,7 @@ def moe_route(x, router_w, top: int, score: str, renormalize: bool,
         pick = probs + correction if correction is not None else probs
     else:
         probs = torch.sigmoid(logits)
-        pick = logits
+        pick = probs + correction if correction is not None else logits
     sel = torch.topk(pick, top, dim=-1).indices
     w = probs.gather(-1, sel)
     if renormalize:
@@ -658,10 +801,13 @@ def moe_route(x, router_w, top: int, score: str, renormalize: bool,
 
 def moe_combine(y, dense, x, experts: int, shared_y=None, shared_gate=None):
     """fp32 [T, W] = sum_e dense[:, e] y[e] over the experts + (sum of the
-    identity outputs' weights) x + sigmoid(shared_gate) shared_y."""
+    identity outputs' weights) x + sigmoid(shared_gate) shared_y (shared_y
+    alone when shared_gate is None)."""
     out = torch.einsum("te,etw->tw", dense[:, :experts], y.float())
     if dense.shape[1] > experts:
         out = out + dense[:, experts:].sum(-1, keepdim=True) * x.float()
-    if shared_y is not None:
+    if shared_y is not None and shared_gate is not None:
         out = out + torch.sigmoid(shared_gate.float()) * shared_y.float()
+    elif shared_y is not None:
+        out = out + shared_y.float()
     return out
