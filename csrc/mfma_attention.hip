@@ -4,7 +4,10 @@
 // head mix and aligned chunks: grouped-query or single-KV-head attention
 // over the paged cache, trailing window with kept first keys, capped
 // scores, denominator sink, values that are the leading entries of the key
-// rows (latent attention: rows of several hundred entries).
+// rows (latent attention: rows of several hundred entries), and pooled
+// blocks behind the window (one mean key/value per block of `pool` positions
+// that lies wholly before a query's window, read from a pooled cache that
+// shares the pages of the key/value cache).
 //
 // A workgroup (4 waves) owns 32 rows = (tokens of consecutive batch rows) x
 // (query heads of one KV head), so one staged key tile serves all of them.
@@ -41,7 +44,17 @@ struct MfOpt {
   const float* sink_vals;
   int vr;        // elements per row of the value cache
   int v_in_k;    // values are read from the key rows
+  const unsigned short* kp;  // pooled keys [NB, G, pr, D] (nullptr: none)
+  const unsigned short* vp;  // pooled values [NB, G, pr, DV]
+  int pool;      // positions per pooled block
+  int pr;        // pooled rows per page
 };
+
+// Pooled blocks a query at position pos sees behind its window.
+PS_DEV int mf_pool_count(int pos, int window, int pool) {
+  const int past = pos - window + 1;
+  return (pool > 0 && window > 0 && past > 0) ? past / pool : 0;
+}
 
 // The softmax arithmetic of a tile is repeated by every wave that owns
 // columns of the same rows, and a wave64 instruction takes four cycles, so
@@ -170,6 +183,7 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
   const bool valid = my_i < ntok;  // ntok <= TPB
   const int my_pos = valid ? s_pos[my_i] : 0;
   const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
+  const int my_pool = opt.kp ? mf_pool_count(my_pos, window, opt.pool) : 0;
   const float inv_cap2 = opt.softcap > 0.f ? 2.0f / opt.softcap : 0.f;
   const bool own_sink = sink && ks == 0;
   float m = own_sink ? (opt.sink_vals ? opt.sink_vals[my_head] : 0.f)
@@ -192,23 +206,39 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
     const int* table = block_tables + (size_t)s_seq[rs] * max_blocks;
     const int kmin = window > 0 ? max(0, s_pos[rs] - window + 1) : 0;
     const int kmax = s_pos[re - 1];
-    // kept first keys behind the run's earliest window, then the windows
-    for (int rg = 0; rg < 2; ++rg) {
-      const int ra = rg == 0 ? 0 : kmin;
-      const int rb = rg == 0 ? min(opt.keep_first, kmin) - 1 : kmax;
+    // kept first keys behind the run's earliest window, the pooled blocks
+    // its last row sees, then the windows
+    const int run_pool =
+        opt.kp ? mf_pool_count(s_pos[re - 1], window, opt.pool) : 0;
+    for (int rg = 0; rg < 3; ++rg) {
+      const int ra = rg == 2 ? kmin : 0;
+      const int rb = rg == 0 ? min(opt.keep_first, kmin) - 1
+                             : (rg == 1 ? run_pool - 1 : kmax);
+      const bool pl = rg == 1;
       for (int j0 = ra; j0 <= rb; j0 += 32, ++tile_no) {
         if (tile_no % KS != ks) continue;
         const int nk = min(32, rb + 1 - j0);
         __syncthreads();  // the previous tile is fully consumed
         if (tid < nk) {
           const int j = j0 + tid;
-          const int64_t gb = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
-          s_kbase[tid] = gb * D;
-          s_vbase[tid] = gb * opt.vr;
+          if (pl) {
+            const int p1 = j * opt.pool;
+            const int64_t gb = ((int64_t)table[p1 / BS] * G + g) * opt.pr +
+                               (p1 % BS) / opt.pool;
+            s_kbase[tid] = gb * D;
+            s_vbase[tid] = gb * DV;
+          } else {
+            const int64_t gb =
+                ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
+            s_kbase[tid] = gb * D;
+            s_vbase[tid] = gb * opt.vr;
+          }
         }
         __syncthreads();
-        mf_stage(sK, PK, kc, s_kbase, nk, D, DP, kvec);
-        if (!opt.v_in_k) mf_stage(sV, PV, vc, s_vbase, nk, DV, DVP, vvec);
+        mf_stage(sK, PK, pl ? opt.kp : kc, s_kbase, nk, D, DP, kvec);
+        if (!opt.v_in_k)
+          mf_stage(sV, PV, pl ? opt.vp : vc, s_vbase, nk, DV, DVP,
+                   pl ? DV % 8 == 0 : vvec);
         __syncthreads();
 
         mf_f32x16 st;
@@ -230,8 +260,10 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
           const int j = j0 + kk;
           float sc = st[r] * scale;
           if (opt.softcap > 0.f) sc = mf_cap(sc, opt.softcap, inv_cap2);
-          const bool vis = mine && kk < nk && j <= my_pos &&
-                           (j >= my_lo || j < opt.keep_first);
+          const bool vis =
+              mine && kk < nk &&
+              (pl ? j < my_pool
+                  : (j <= my_pos && (j >= my_lo || j < opt.keep_first)));
           sc = vis ? sc : PS_NEG_INF;
           p[r] = sc;
           mx = fmaxf(mx, sc);
@@ -420,15 +452,22 @@ extern "C" int mx_mfma_attention(
     const void* token_seq, const void* token_pos, int T_, int H, int G, int D,
     int DV, int BS, float scale, int window, int sink, int keep_first,
     float softcap, const void* sink_vals, int vrow, int v_in_k, int splits,
-    void* scratch, int mode, void* stream) {
+    void* scratch, int mode, const void* kpool, const void* vpool, int pool,
+    void* stream) {
   if (T_ <= 0) return 0;
   if (G < 1 || H % G) return 1;
   const int rep = H / G;
   if (rep < 32 ? (32 % rep != 0) : (rep % 32 != 0)) return 1;
   if (DV > 512 || DV < 1 || D < 1 || vrow < DV) return 1;
   if (v_in_k && DV > D) return 1;
+  const bool pooled = kpool != nullptr && pool > 0 && window > 0;
+  if (pooled && v_in_k) return 1;
   const MfOpt opt = {keep_first > 0 ? keep_first : 0, softcap,
-                     (const float*)sink_vals, vrow, v_in_k ? 1 : 0};
+                     (const float*)sink_vals, vrow, v_in_k ? 1 : 0,
+                     pooled ? (const unsigned short*)kpool : nullptr,
+                     pooled ? (const unsigned short*)vpool : nullptr,
+                     pooled ? pool : 0,
+                     pooled ? (BS + pool - 1) / pool : 0};
   int KS = splits > 1 && scratch != nullptr ? splits : 1;
   const int cbw = ((DV + 31) / 32 + 3) / 4;
 #define MF_GO(N)                                                             \

@@ -6,17 +6,24 @@
 //                    of the queries' rotary parts, paged append of
 //                    [latent | key part], assembly of the latent-space
 //                    queries;
+//   pool_append      mean key/value of every block of positions a step
+//                    completes, into the pooled caches;
 //   short_conv_silu  causal per-channel convolution over time + silu with
 //                    the last taps-1 inputs of every sequence as state.
 // All arithmetic is fp32; the element type decides loads and the final
 // rounding.
 #include "mix_common.h"
 
-// One wave per head: x / sqrt(mean(x^2) + eps) * w over D entries, then the
-// first rot_dims entries turn in interleaved pairs (2i, 2i+1) by row
-// `position` of the table cs [table_rows][rot_dims / 2][cos, sin]. A lane
-// reads its own entry and its pair partner's (a neighbouring lane's) before
-// it stores, and the wave runs in step, so the query is rewritten in place.
+// One wave per head: x / sqrt(mean(x^2) + eps) * w over D entries (the mean
+// over the head, or with norm_all over the whole query / key projection,
+// whose weights then have H*D / G*D entries), then the first rot_dims
+// entries turn by row `position` of the table cs [table_rows][rot_dims / 2]
+// [cos, sin]: interleaved pairs (2i, 2i+1), or with `half` pairs (i, i +
+// rot_dims / 2). A lane reads its own entries and their pair partners' and
+// only then stores, and the wave runs in step, so the query is rewritten in
+// place. Heads of up to 64 * AP_MAX_PER_LANE entries.
+#define AP_MAX_PER_LANE 8
+
 template <typename T>
 __global__ __launch_bounds__(256) void attn_prep_kernel(
     T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk,
@@ -25,7 +32,9 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
     const T* __restrict__ vfirst, int ldvf, T* __restrict__ kc,
     T* __restrict__ vc, const int64_t* __restrict__ slots, int H, int G,
     int D, int DV, int BS, const float* __restrict__ cs, int table_rows,
-    int rot_dims, const int* __restrict__ positions) {
+    int rot_dims, const int* __restrict__ positions, int norm_all,
+    int half) {
+  __shared__ float red[17];
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
@@ -35,14 +44,37 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
   const int64_t slot = slots[t];
   const int64_t blk = slot >= 0 ? slot / BS : 0;
   const int off = slot >= 0 ? (int)(slot % BS) : 0;
+  // whole-projection norms: one sum of squares over all query entries and
+  // one over all key entries
+  float inv_q = 1.f, inv_k = 1.f;
+  if (norm_all && qw != nullptr) {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H * D; c += blockDim.x) {
+      const float x = MxElem<T>::ld(q + (size_t)t * ldq + c);
+      ss += x * x;
+    }
+    inv_q = 1.0f / sqrtf(mx_block_sum(ss, red) / (float)(H * D) + eps);
+  }
+  if (norm_all && kw != nullptr) {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < G * D; c += blockDim.x) {
+      const float x = MxElem<T>::ld(k + (size_t)t * ldk + c);
+      ss += x * x;
+    }
+    inv_k = 1.0f / sqrtf(mx_block_sum(ss, red) / (float)(G * D) + eps);
+  }
+  const int hd = rot_dims >> 1;
   for (int hh = wave; hh < H + G; hh += nw) {
     const bool is_q = hh < H;
     const int g = hh - H;
     const T* src = is_q ? q + (size_t)t * ldq + hh * D
                         : k + (size_t)t * ldk + g * D;
     const float* wgt = is_q ? qw : kw;
-    float inv = 1.f;
-    if (wgt != nullptr) {
+    // weight row of this head
+    const float* wr =
+        wgt != nullptr && norm_all ? wgt + (is_q ? hh : g) * D : wgt;
+    float inv = is_q ? inv_q : inv_k;
+    if (wgt != nullptr && !norm_all) {
       float ss = 0.f;
       for (int d = lane; d < D; d += 64) {
         const float x = MxElem<T>::ld(src + d);
@@ -58,16 +90,31 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
       dst = kc + ((blk * G + g) * BS + off) * (int64_t)D;
     }
     if (dst != nullptr) {
-      for (int d = lane; d < D; d += 64) {
-        float x = MxElem<T>::ld(src + d);
-        if (wgt != nullptr) x *= inv * wgt[d];
-        if (csr != nullptr && d < rot_dims) {
-          float y = MxElem<T>::ld(src + (d ^ 1));
-          if (wgt != nullptr) y *= inv * wgt[d ^ 1];
-          const float* e = csr + (d & ~1);
-          x = (d & 1) ? x * e[0] + y * e[1] : x * e[0] - y * e[1];
+      float res[AP_MAX_PER_LANE];
+#pragma unroll
+      for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) {
+          float x = MxElem<T>::ld(src + d);
+          if (wgt != nullptr) x *= inv * wr[d];
+          if (csr != nullptr && d < rot_dims) {
+            // partner entry and whether this entry is the pair's first
+            const int pd = half ? (d < hd ? d + hd : d - hd) : (d ^ 1);
+            const bool first = half ? d < hd : (d & 1) == 0;
+            const int pi = half ? (d < hd ? d : d - hd) : (d >> 1);
+            float y = MxElem<T>::ld(src + pd);
+            if (wgt != nullptr) y *= inv * wr[pd];
+            const float* e = csr + 2 * pi;
+            x = first ? x * e[0] - y * e[1] : x * e[0] + y * e[1];
+          }
+          res[i] = x;
         }
-        MxElem<T>::st(dst + d, x);
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) MxElem<T>::st(dst + d, res[i]);
       }
     }
   }
@@ -82,6 +129,42 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
       const int g = c / DV, d = c % DV;
       MxElem<T>::st(vc + ((blk * G + g) * BS + off) * (int64_t)DV + d, x);
     }
+  }
+}
+
+// Pooled keys/values: workgroup (segment, i) takes the i-th block of `pool`
+// positions whose last position this step appended (block b covers b*pool
+// .. b*pool + pool - 1) and stores the fp32 means of its cached keys and
+// values, rounded to the cache type, in the pooled caches [NB, G, pr, D|DV]:
+// in the page of the block's first position, at row (first position mod BS)
+// div pool.
+template <typename T>
+__global__ __launch_bounds__(256) void pool_append_kernel(
+    const T* __restrict__ kc, const T* __restrict__ vc, T* __restrict__ kp,
+    T* __restrict__ vp, const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ seq_rows, int G, int D, int DV, int BS, int pool,
+    int pr) {
+  const int* sr = seq_rows + 4 * blockIdx.x;
+  const int n = sr[1], p0 = sr[2];
+  const int b = p0 / pool + blockIdx.y;
+  if (b >= (p0 + n) / pool) return;
+  const int* table = block_tables + (size_t)blockIdx.x * max_blocks;
+  const int first = b * pool;
+  const int64_t prow_base = (int64_t)table[first / BS] * G;
+  const int prow = (first % BS) / pool;
+  const float cnt = (float)pool;
+  for (int c = threadIdx.x; c < G * (D + DV); c += blockDim.x) {
+    const bool is_k = c < G * D;
+    const int cc = is_k ? c : c - G * D;
+    const int w = is_k ? D : DV;
+    const int g = cc / w, d = cc - g * w;
+    const T* cache = is_k ? kc : vc;
+    float acc = 0.f;
+    for (int j = first; j < first + pool; ++j)
+      acc += MxElem<T>::ld(
+          cache + (((int64_t)table[j / BS] * G + g) * BS + (j % BS)) * w + d);
+    T* dst = (is_k ? kp : vp) + ((prow_base + g) * pr + prow) * (int64_t)w + d;
+    MxElem<T>::st(dst, acc / cnt);
   }
 }
 
@@ -219,7 +302,8 @@ void mx_attn_prep(void* q, int ldq, const void* k, int ldk, void* v, int ldv,
                   const void* vfirst, int ldvf, void* kc, void* vc,
                   const void* slots, int T_, int H, int G, int D, int DV,
                   int BS, const void* cos_sin, int table_rows, int rot_dims,
-                  const void* positions, int dtype, void* stream) {
+                  const void* positions, int norm_all, int half, int dtype,
+                  void* stream) {
   if (T_ <= 0) return;
   MX_DISPATCH_DTYPE(dtype, {
     hipLaunchKernelGGL((attn_prep_kernel<T>), dim3(T_), dim3(256), 0,
@@ -228,7 +312,23 @@ void mx_attn_prep(void* q, int ldq, const void* k, int ldk, void* v, int ldv,
                        (const float*)vmix, (const T*)vfirst, ldvf, (T*)kc,
                        (T*)vc, (const int64_t*)slots, H, G, D, DV, BS,
                        (const float*)cos_sin, table_rows, rot_dims,
-                       (const int*)positions);
+                       (const int*)positions, norm_all, half);
+  })
+}
+
+void mx_pool_append(const void* kc, const void* vc, void* kp, void* vp,
+                    const void* block_tables, int max_blocks,
+                    const void* seq_rows, int S_, int blocks_per_seg, int G,
+                    int D, int DV, int BS, int pool, int dtype,
+                    void* stream) {
+  if (S_ <= 0 || blocks_per_seg <= 0 || pool < 1) return;
+  const int pr = (BS + pool - 1) / pool;
+  MX_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((pool_append_kernel<T>), dim3(S_, blocks_per_seg),
+                       dim3(256), 0, (hipStream_t)stream, (const T*)kc,
+                       (const T*)vc, (T*)kp, (T*)vp,
+                       (const int*)block_tables, max_blocks,
+                       (const int*)seq_rows, G, D, DV, BS, pool, pr);
   })
 }
 

@@ -1,9 +1,10 @@
 // Router of a routed feed-forward, one kernel per layer and step:
 //   logits = W_router x            (fp32 accumulation of the inputs' products)
 //   scores = softmax(logits)  |  sigmoid(logits)
-//   choice = the `top` largest of scores + correction (softmax; the
-//            correction only moves the choice) or of the logits (sigmoid:
-//            the fp32 sigmoid saturates and would tie large scores)
+//   choice = the `top` largest of scores + correction (the correction only
+//            moves the choice); sigmoid scores without a correction are
+//            ranked by their logits (the fp32 sigmoid saturates and would
+//            tie large scores)
 //   weights = the chosen scores, divided by (their sum + renorm_eps) when
 //            asked, times scale
 // Outputs: the chosen outputs' indices and weights [T, top] (best first) and
@@ -86,8 +87,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
   if (sigmoid_scores) {
     for (int e = lane; e < n_out; e += 64) {
       const float z = score[e];
-      pick[e] = z;
-      score[e] = mx_sigmoid(z);
+      const float sg = mx_sigmoid(z);
+      pick[e] = corr != nullptr ? sg + corr[e] : z;
+      score[e] = sg;
     }
   } else {
     float m = -INFINITY;
@@ -147,7 +149,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
 // Weighted sum of the all-experts path: y [E][T][W] holds every expert's
 // output for every row; out[t] = sum_e dense[t][e] y[e][t] (experts a row did
 // not choose have weight 0 and are not read) + (sum of the identity outputs'
-// weights) x[t] + sigmoid(sgate[t]) ys[t] (shared expert, optional). fp32 out.
+// weights) x[t] + sigmoid(sgate[t]) ys[t] (shared expert, optional; without
+// sgate it joins unscaled). fp32 out.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(
     float* __restrict__ out, const T* __restrict__ y,
@@ -167,7 +170,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
   for (int e = E; e < n_out; ++e) wid += dw[e];
   if (wid != 0.f) acc += wid * MxElem<T>::ld(x + (size_t)t * ldx + c);
   if (ys != nullptr)
-    acc += mx_sigmoid(MxElem<T>::ld(sgate + (size_t)t * ldsg)) *
+    acc += (sgate != nullptr
+                ? mx_sigmoid(MxElem<T>::ld(sgate + (size_t)t * ldsg))
+                : 1.f) *
            MxElem<T>::ld(ys + (size_t)t * ldys + c);
   out[(size_t)t * W + c] = acc;
 }

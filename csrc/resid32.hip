@@ -128,6 +128,9 @@ __global__ __launch_bounds__(256) void depth_mix_kernel(
 #define MX_ACT_GELU_TANH 1
 #define MX_ACT_CLAMPED_SWISH 2
 #define MX_ACT_SIGMOID 3  // sigmoid(g) * u: an output gate
+#define MX_ACT_RELU2 4    // relu(g)^2 * u
+// up == nullptr: the plain activation (u = 1; the clamped form then has no
+// second factor)
 
 template <typename T, int KIND>
 __global__ __launch_bounds__(256) void gated_act_kernel(
@@ -137,9 +140,12 @@ __global__ __launch_bounds__(256) void gated_act_kernel(
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= F) return;
   float g = MxElem<T>::ld(gate + (size_t)t * ldg + c);
-  float u = MxElem<T>::ld(up + (size_t)t * ldu + c);
+  float u = up != nullptr ? MxElem<T>::ld(up + (size_t)t * ldu + c) : 1.f;
   float y;
-  if (KIND == MX_ACT_SILU) {
+  if (KIND == MX_ACT_RELU2) {
+    const float r = fmaxf(g, 0.f);
+    y = r * r * u;
+  } else if (KIND == MX_ACT_SILU) {
     y = g * mx_sigmoid(g) * u;
   } else if (KIND == MX_ACT_GELU_TANH) {
     const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
@@ -148,7 +154,7 @@ __global__ __launch_bounds__(256) void gated_act_kernel(
     y = mx_sigmoid(g) * u;
   } else {
     g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
+    u = up != nullptr ? fminf(fmaxf(u, -limit), limit) : 0.f;
     y = g * mx_sigmoid(1.702f * g) * (u + 1.0f);
   }
   MxElem<T>::st(out + (size_t)t * ldo + c, y);
@@ -164,7 +170,11 @@ __global__ __launch_bounds__(256) void gated_act_bf16x8_kernel(
   const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (c >= F) return;
   const uint4 gq = *(const uint4*)(gate + (size_t)t * ldg + c);
-  const uint4 uq = *(const uint4*)(up + (size_t)t * ldu + c);
+  // without `up` every factor is 1.0 (bf16 0x3f80)
+  const uint4 uq = up != nullptr
+                       ? *(const uint4*)(up + (size_t)t * ldu + c)
+                       : make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u,
+                                    0x3f803f80u);
   const unsigned int gw[4] = {gq.x, gq.y, gq.z, gq.w};
   const unsigned int uw[4] = {uq.x, uq.y, uq.z, uq.w};
   unsigned int ow[4];
@@ -175,7 +185,10 @@ __global__ __launch_bounds__(256) void gated_act_bf16x8_kernel(
     for (int e = 0; e < 2; ++e) {
       float g = __uint_as_float(e ? (gw[k] & 0xffff0000u) : (gw[k] << 16));
       float u = __uint_as_float(e ? (uw[k] & 0xffff0000u) : (uw[k] << 16));
-      if (KIND == MX_ACT_SILU) {
+      if (KIND == MX_ACT_RELU2) {
+        const float r = fmaxf(g, 0.f);
+        y[e] = r * r * u;
+      } else if (KIND == MX_ACT_SILU) {
         y[e] = g * mx_sigmoid(g) * u;
       } else if (KIND == MX_ACT_GELU_TANH) {
         const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
@@ -184,7 +197,7 @@ __global__ __launch_bounds__(256) void gated_act_bf16x8_kernel(
         y[e] = mx_sigmoid(g) * u;
       } else {
         g = fminf(g, limit);
-        u = fminf(fmaxf(u, -limit), limit);
+        u = up != nullptr ? fminf(fmaxf(u, -limit), limit) : 0.f;
         y[e] = g * mx_sigmoid(1.702f * g) * (u + 1.0f);
       }
     }
@@ -355,7 +368,11 @@ void mx_gated_act(void* out, int ldo, const void* gate, int ldg,
       (((size_t)out | (size_t)gate | (size_t)up) & 15) == 0) {
     dim3 grid8((F / 8 + 255) / 256, T_);
     typedef unsigned short U;
-    if (kind == MX_ACT_SILU) {
+    if (kind == MX_ACT_RELU2) {
+      hipLaunchKernelGGL((gated_act_bf16x8_kernel<MX_ACT_RELU2>), grid8,
+                         dim3(256), 0, (hipStream_t)stream, (U*)out, ldo,
+                         (const U*)gate, ldg, (const U*)up, ldu, F, limit);
+    } else if (kind == MX_ACT_SILU) {
       hipLaunchKernelGGL((gated_act_bf16x8_kernel<MX_ACT_SILU>), grid8,
                          dim3(256), 0, (hipStream_t)stream, (U*)out, ldo,
                          (const U*)gate, ldg, (const U*)up, ldu, F, limit);
@@ -377,7 +394,11 @@ void mx_gated_act(void* out, int ldo, const void* gate, int ldg,
   }
   dim3 grid((F + 255) / 256, T_);
   MX_DISPATCH_DTYPE(dtype, {
-    if (kind == MX_ACT_SILU) {
+    if (kind == MX_ACT_RELU2) {
+      hipLaunchKernelGGL((gated_act_kernel<T, MX_ACT_RELU2>), grid, dim3(256),
+                         0, (hipStream_t)stream, (T*)out, ldo,
+                         (const T*)gate, ldg, (const T*)up, ldu, F, limit);
+    } else if (kind == MX_ACT_SILU) {
       hipLaunchKernelGGL((gated_act_kernel<T, MX_ACT_SILU>), grid, dim3(256),
                          0, (hipStream_t)stream, (T*)out, ldo,
                          (const T*)gate, ldg, (const T*)up, ldu, F, limit);

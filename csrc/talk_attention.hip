@@ -3,7 +3,13 @@
 // visible behind the window), capped scores and an optional denominator
 // sink (score 0 or a learned per-head score). The values may be the leading
 // entries of wider cache rows, so keys that carry their values (latent
-// attention) need one cache.
+// attention) need one cache. With a window, blocks of `pool` consecutive
+// positions that lie wholly before a query's window can stay visible through
+// one pooled key/value each (TaOpt::kp / vp): block b is seen by a query at
+// position p when (b + 1) * pool <= p - window + 1, and lives in the page of
+// its first position at row (first position mod BS) div pool of a pooled
+// cache with ceil(BS / pool) rows per page. The kernels walk three key
+// ranges in turn: kept first keys, pooled blocks, window.
 //
 // One launch covers a ragged batch: every token carries (its sequence's
 // block-table row, its position); keys and values come from the paged
@@ -28,7 +34,25 @@ struct TaOpt {
   float softcap;
   const float* sink_vals;
   int vr;
+  const void* kp;  // pooled keys [NB, G, pr, D] (nullptr: none)
+  const void* vp;  // pooled values [NB, G, pr, DV]
+  int pool;        // positions per pooled block
+  int pr;          // pooled rows per page
 };
+
+// Pooled blocks a query at position pos sees behind its window.
+PS_DEV int ta_pool_count(int pos, int window, int pool) {
+  const int past = pos - window + 1;  // positions before the window
+  return (pool > 0 && window > 0 && past > 0) ? past / pool : 0;
+}
+
+// Row of key j in a paged cache with R rows per page, each row standing for
+// P positions (the key/value cache: P = 1, R = BS).
+PS_DEV int64_t ta_row(const int* __restrict__ table, int j, int G, int g,
+                      int BS, int P, int R) {
+  const int pos = j * P;
+  return ((int64_t)table[pos / BS] * G + g) * R + (pos % BS) / P;
+}
 
 PS_DEV float ta_cap(float sc, float cap) {
   return cap > 0.f ? cap * tanhf(sc / cap) : sc;
@@ -91,19 +115,25 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
   }
   __syncthreads();
 
-  // two key ranges: the kept first keys behind the window, then the window
-  for (int rg = 0; rg < 2; ++rg) {
-  const int ra = rg == 0 ? 0 : lo;
-  const int rb = rg == 0 ? min(opt.keep_first, lo) - 1 : pos;
+  // key ranges: the kept first keys behind the window, the pooled blocks
+  // behind it, then the window
+  const int npool = opt.kp ? ta_pool_count(pos, window, opt.pool) : 0;
+  for (int rg = 0; rg < 3; ++rg) {
+  const int ra = rg == 2 ? lo : 0;
+  const int rb = rg == 0 ? min(opt.keep_first, lo) - 1
+                         : (rg == 1 ? npool - 1 : pos);
+  const T* kcr = rg == 1 ? (const T*)opt.kp : kc;
+  const T* vcr = rg == 1 ? (const T*)opt.vp : vc;
+  const int cP = rg == 1 ? opt.pool : 1, cR = rg == 1 ? opt.pr : BS;
+  const int cvr = rg == 1 ? DV : opt.vr;
   for (int j0 = ra; j0 <= rb; j0 += TA_KT) {
     const int nk = min(TA_KT, rb + 1 - j0);
     // raw scores of every (head, key) pair of the tile
     for (int it = threadIdx.x; it < H * nk; it += blockDim.x) {
       const int jj = it / H, h = it % H;
       const int j = j0 + jj;
-      const int64_t blk = table[j / BS];
       const T* kr =
-          kc + ((blk * G + (h0 + h) / rep) * BS + (j % BS)) * (int64_t)D;
+          kcr + ta_row(table, j, G, (h0 + h) / rep, BS, cP, cR) * (int64_t)D;
       const float* qh = sq + h * D;
       float acc = 0.f;
       for (int d = 0; d < D; ++d) acc += qh[d] * MxElem<T>::ld(kr + d);
@@ -147,10 +177,9 @@ __global__ __launch_bounds__(256) void talk_attn_kernel(
       float acc = sacc[it] * sal[h];
       for (int jj = 0; jj < nk; ++jj) {
         const int j = j0 + jj;
-        const int64_t blk = table[j / BS];
         acc += sp[h * TA_KT + jj] *
-               MxElem<T>::ld(vc + ((blk * G + gk) * BS + (j % BS)) *
-                                      (int64_t)opt.vr + d);
+               MxElem<T>::ld(vcr + ta_row(table, j, G, gk, BS, cP, cR) *
+                                       (int64_t)cvr + d);
       }
       sacc[it] = acc;
     }
@@ -196,7 +225,8 @@ struct TaVec<mx_bf16> {
 template <typename T, int DP, int PITCH>
 PS_DEV void ta_stage(float* __restrict__ sdst, const T* __restrict__ cache,
                      const int* __restrict__ table, int j0, int nk, int G,
-                     int Dw, int BS, int RW) {
+                     int Dw, int BS, int RW, int P = 1, int R = 0) {
+  if (R == 0) R = BS;
   // Dw elements of every cache row of RW elements are staged
   constexpr int VEC = TaVec<T>::N;
   constexpr int U = 8;
@@ -215,7 +245,7 @@ PS_DEV void ta_stage(float* __restrict__ sdst, const T* __restrict__ cache,
           const int row = idx / vpr, c = idx - row * vpr;
           const int jj = row / G, g = row - jj * G;
           const int j = j0 + jj;
-          const int64_t gb = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
+          const int64_t gb = ta_row(table, j, G, g, BS, P, R);
           buf[u] = *(const float4*)(cache + gb * RW + c * VEC);
           off[u] = row * PITCH + c * VEC;
         }
@@ -236,7 +266,7 @@ PS_DEV void ta_stage(float* __restrict__ sdst, const T* __restrict__ cache,
       const int d = e % DP, row = e / DP;
       const int jj = row / G, g = row - jj * G;
       const int j = j0 + jj;
-      const int64_t gb = ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
+      const int64_t gb = ta_row(table, j, G, g, BS, P, R);
       sdst[row * PITCH + d] = d < Dw ? MxElem<T>::ld(cache + gb * RW + d) : 0.f;
     }
   }
@@ -304,6 +334,7 @@ __global__ __launch_bounds__(256) void talk_attn_tiled_kernel(
   int my_lo = 0;
   if (chunk > 0) my_lo = (my_pos / chunk) * chunk;
   if (window > 0) my_lo = max(my_lo, my_pos - window + 1);
+  const int my_pool = opt.kp ? ta_pool_count(my_pos, window, opt.pool) : 0;
 
   int rs = 0;
   while (rs < nrows) {
@@ -318,15 +349,26 @@ __global__ __launch_bounds__(256) void talk_attn_tiled_kernel(
     if (window > 0) kmin = max(kmin, s_pos[rs] - window + 1);
     const int kmax = s_pos[re - 1];
 
-    // kept first keys behind the run's earliest window, then the windows
-    for (int rg = 0; rg < 2; ++rg) {
-    const int ra = rg == 0 ? 0 : kmin;
-    const int rb = rg == 0 ? min(opt.keep_first, kmin) - 1 : kmax;
+    // kept first keys behind the run's earliest window, the pooled blocks
+    // its last row sees, then the windows
+    const int run_pool =
+        opt.kp ? ta_pool_count(s_pos[re - 1], window, opt.pool) : 0;
+    for (int rg = 0; rg < 3; ++rg) {
+    const int ra = rg == 2 ? kmin : 0;
+    const int rb = rg == 0 ? min(opt.keep_first, kmin) - 1
+                           : (rg == 1 ? run_pool - 1 : kmax);
     for (int j0 = ra; j0 <= rb; j0 += KT) {
       const int nk = min(KT, rb + 1 - j0);
       __syncthreads();  // the previous tile is fully consumed
-      ta_stage<T, DP, DP>(sK, kc, table, j0, nk, G, D, BS, D);
-      ta_stage<T, DP, DP>(sV, vc, table, j0, nk, G, DV, BS, opt.vr);
+      if (rg == 1) {
+        ta_stage<T, DP, DP>(sK, (const T*)opt.kp, table, j0, nk, G, D, BS, D,
+                            opt.pool, opt.pr);
+        ta_stage<T, DP, DP>(sV, (const T*)opt.vp, table, j0, nk, G, DV, BS,
+                            DV, opt.pool, opt.pr);
+      } else {
+        ta_stage<T, DP, DP>(sK, kc, table, j0, nk, G, D, BS, D);
+        ta_stage<T, DP, DP>(sV, vc, table, j0, nk, G, DV, BS, opt.vr);
+      }
       __syncthreads();
       if (mine) {
         for (int jj = 0; jj < nk; ++jj) {
@@ -358,7 +400,8 @@ __global__ __launch_bounds__(256) void talk_attn_tiled_kernel(
           }
           sc = ta_cap(sc, opt.softcap);
           const int j = j0 + jj;
-          if (j > my_pos || (j < my_lo && j >= opt.keep_first))
+          if (rg == 1 ? j >= my_pool
+                      : (j > my_pos || (j < my_lo && j >= opt.keep_first)))
             sc = PS_NEG_INF;
           sM[jj * NP + tid] = sc;
           mx = fmaxf(mx, sc);
@@ -470,8 +513,11 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
   int lo = 0, pos = token_pos[t];
   if (chunk > 0) lo = (pos / chunk) * chunk;
   if (window > 0) lo = max(lo, pos - window + 1);
-  // the kept first keys behind the window go to share 0
+  // the kept first keys and the pooled blocks behind the window go to
+  // share 0
   const int kept = ks == 0 ? min(opt.keep_first, lo) : 0;
+  const int npool =
+      (ks == 0 && opt.kp) ? ta_pool_count(pos, window, opt.pool) : 0;
   if (KS > 1) {
     // this workgroup's share of the visible keys, in whole tiles
     const int tiles = (pos + 1 - lo + TK - 1) / TK;
@@ -498,14 +544,21 @@ __global__ __launch_bounds__(256) void talk_attn_split_kernel(
                      : PS_NEG_INF;
   float l = own_sink ? 1.f : 0.f;
 
-  for (int rg = 0; rg < 2; ++rg) {
-  const int ra = rg == 0 ? 0 : lo;
-  const int rb = rg == 0 ? kept - 1 : pos;
+  for (int rg = 0; rg < 3; ++rg) {
+  const int ra = rg == 2 ? lo : 0;
+  const int rb = rg == 0 ? kept - 1 : (rg == 1 ? npool - 1 : pos);
   for (int j0 = ra; j0 <= rb; j0 += TK) {
     const int nk = min(TK, rb + 1 - j0);
     __syncthreads();
-    ta_stage<T, DP, PITCH>(sK, kc, table, j0, nk, G, D, BS, D);
-    ta_stage<T, DP, PITCH>(sV, vc, table, j0, nk, G, DV, BS, opt.vr);
+    if (rg == 1) {
+      ta_stage<T, DP, PITCH>(sK, (const T*)opt.kp, table, j0, nk, G, D, BS, D,
+                             opt.pool, opt.pr);
+      ta_stage<T, DP, PITCH>(sV, (const T*)opt.vp, table, j0, nk, G, DV, BS,
+                             DV, opt.pool, opt.pr);
+    } else {
+      ta_stage<T, DP, PITCH>(sK, kc, table, j0, nk, G, D, BS, D);
+      ta_stage<T, DP, PITCH>(sV, vc, table, j0, nk, G, DV, BS, opt.vr);
+    }
     __syncthreads();
     if (valid) {
       for (int c = 0; c < KPT; ++c) {
@@ -706,11 +759,15 @@ extern "C" int mx_talk_attention(void* out, int ldout, const void* q,
                                  int sink, int dtype, int variant,
                                  int splits, void* scratch, int keep_first,
                                  float softcap, const void* sink_vals,
-                                 int vrow, void* stream) {
+                                 int vrow, const void* kpool,
+                                 const void* vpool, int pool, void* stream) {
   if (T_ <= 0) return 0;
   if (vrow < DV) return 3;
+  const bool pooled = kpool != nullptr && pool > 0 && window > 0;
   const TaOpt opt = {keep_first > 0 ? keep_first : 0, softcap,
-                     (const float*)sink_vals, vrow};
+                     (const float*)sink_vals, vrow,
+                     pooled ? kpool : nullptr, pooled ? vpool : nullptr,
+                     pooled ? pool : 0, pooled ? (BS + pool - 1) / pool : 0};
   const int dmax = D > DV ? D : DV;
   if ((variant == 0 || variant == 2) && H <= 256 && dmax <= 128) {
     int rc = 1;

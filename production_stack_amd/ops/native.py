@@ -1,14 +1,19 @@
-"""Builder and loader of the mixer-kernel library (`_mixops.so`).
+"""Builder and loader of the mixer-kernel libraries (`_mixops*.so`).
 
-The fp32-residual / delta-rule / linear-scan / attention kernels
-(csrc/resid32.hip, csrc/delta_rule.hip, csrc/gated_delta.hip,
-csrc/linear_scan.hip, csrc/talk_attention.hip, csrc/mixer_prep.hip,
-csrc/mfma_attention.hip, csrc/moe_route.hip) expose a plain C ABI, so the
-library needs hipcc only: no torch headers, seconds-to-minutes to build, and
-a fresh checkout can compile just these files on first use without building
-the large `_C` extension. Launchers receive raw device pointers and the
-current HIP stream; shape checks live in the Python wrappers
+The fp32-residual / delta-rule / linear-scan / attention kernels expose a
+plain C ABI, so the libraries need hipcc only: no torch headers,
+seconds-to-minutes to build, and a fresh checkout compiles on first use just
+the group of files a model's ops live in, without building the large `_C`
+extension. Launchers receive raw device pointers and the current HIP stream;
+shape checks live in the Python wrappers
 (production_stack_amd/ops/__init__.py).
+
+Groups (one shared library each):
+  core    resid32, norm_conv, mixer_prep, talk_attention, mfma_attention,
+          moe_route, mingru_scan            -> _mixops.so
+  delta   delta_rule                        -> _mixops_delta.so
+  gdelta  gated_delta                       -> _mixops_gdelta.so
+  scan    linear_scan                       -> _mixops_scan.so
 """
 
 from __future__ import annotations
@@ -30,39 +35,66 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
-# (source, extra defines): the delta-rule file is compiled once per element
-# type so its many head-size instantiations build in parallel
-UNITS = [
-    ("resid32.hip", []),
-    ("talk_attention.hip", []),
-    ("delta_rule.hip", ["-DMX_ONLY_DTYPE=0"]),
-    ("delta_rule.hip", ["-DMX_ONLY_DTYPE=1"]),
-    ("mixer_prep.hip", []),
-    ("mfma_attention.hip", []),
-    ("moe_route.hip", []),
-    ("gated_delta.hip", ["-DMX_ONLY_DTYPE=0"]),
-    ("gated_delta.hip", ["-DMX_ONLY_DTYPE=1"]),
+# group -> [(source, extra defines)]: the recurrence files are compiled once
+# per element type (or decay law) so their many head-size instantiations
+# build in parallel
+GROUPS = {
+    "core": [
+        ("resid32.hip", []),
+        ("norm_conv.hip", []),
+        ("talk_attention.hip", []),
+        ("mixer_prep.hip", []),
+        ("mfma_attention.hip", []),
+        ("moe_route.hip", []),
+        ("mingru_scan.hip", []),
+    ],
+    "delta": [
+        ("delta_rule.hip", ["-DMX_ONLY_DTYPE=0"]),
+        ("delta_rule.hip", ["-DMX_ONLY_DTYPE=1"]),
+    ],
+    "gdelta": [
+        ("gated_delta.hip", ["-DMX_ONLY_DTYPE=0"]),
+        ("gated_delta.hip", ["-DMX_ONLY_DTYPE=1"]),
+    ],
     # one unit per (decay law, element type)
-    *[("linear_scan.hip", [f"-DLS_ONLY={i}"]) for i in range(6)],
-]
+    "scan": [("linear_scan.hip", [f"-DLS_ONLY={i}"]) for i in range(6)],
+}
 
-_lib = None
+LIB_PATHS = {
+    "core": LIB_PATH,
+    "delta": os.path.join(PKG, "_mixops_delta.so"),
+    "gdelta": os.path.join(PKG, "_mixops_gdelta.so"),
+    "scan": os.path.join(PKG, "_mixops_scan.so"),
+}
+
+# entry points outside the core group
+SYMBOL_GROUP = {
+    "mx_delta_rule": "delta",
+    "mx_gated_delta": "gdelta",
+    "mx_linear_scan": "scan",
+    "mx_linear_scan_splits": "scan",
+}
+
+# entry points that return a status (the others return nothing)
+INT_RESULT = {
+    "mx_delta_rule", "mx_talk_attention", "mx_gated_delta",
+    "mx_short_conv_silu", "mx_mfma_attention", "mx_linear_scan",
+    "mx_linear_scan_splits", "mx_norm_conv32", "mx_moe_route",
+}
 
 
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
-        raise RuntimeError("hipcc not found: cannot build _mixops.so")
+        raise RuntimeError("hipcc not found: cannot build the mixer kernels")
     return exe
 
 
-def build(force: bool = False) -> str:
-    """Compile the library in-tree (atomic replace). Returns its path."""
-    if os.path.exists(LIB_PATH) and not force:
-        return LIB_PATH
+def _build_group(group: str) -> str:
     hipcc = _hipcc()
     src_dir = os.path.join(ROOT, "csrc")
-    tmp = tempfile.mkdtemp(prefix="mixops-", dir=PKG)
+    units = GROUPS[group]
+    tmp = tempfile.mkdtemp(prefix=f"mixops-{group}-", dir=PKG)
     try:
         def compile_one(i_unit):
             i, (src, defs) = i_unit
@@ -76,8 +108,8 @@ def build(force: bool = False) -> str:
                     f"hipcc failed on {src}:\n{r.stdout[-4000:]}")
             return obj
 
-        with ThreadPoolExecutor(max_workers=len(UNITS)) as ex:
-            objs = list(ex.map(compile_one, enumerate(UNITS)))
+        with ThreadPoolExecutor(max_workers=len(units)) as ex:
+            objs = list(ex.map(compile_one, enumerate(units)))
         out = os.path.join(tmp, "lib.so")
         r = subprocess.run(
             [hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objs,
@@ -85,35 +117,57 @@ def build(force: bool = False) -> str:
             stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"link failed:\n{r.stdout[-4000:]}")
-        os.replace(out, LIB_PATH)
+        os.replace(out, LIB_PATHS[group])
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+    return LIB_PATHS[group]
+
+
+def build(force: bool = False, groups=None) -> str:
+    """Compile the libraries in-tree (atomic replace), all groups unless
+    `groups` names some. Returns the core library's path."""
+    todo = [g for g in (groups or GROUPS)
+            if force or not os.path.exists(LIB_PATHS[g])]
+    with ThreadPoolExecutor(max_workers=max(len(todo), 1)) as ex:
+        list(ex.map(_build_group, todo))
     return LIB_PATH
 
 
+class _Libs:
+    """Attribute access resolves an entry point in its group's library,
+    which is loaded (and built, when nothing is built) on first use."""
+
+    def __init__(self) -> None:
+        self._handles = {}
+
+    def _handle(self, group: str):
+        h = self._handles.get(group)
+        if h is None:
+            if not os.path.exists(LIB_PATHS[group]):
+                _build_group(group)
+            h = ctypes.CDLL(LIB_PATHS[group])
+            self._handles[group] = h
+        return h
+
+    def __getattr__(self, name: str):
+        if not name.startswith("mx_"):
+            raise AttributeError(name)
+        fn = getattr(self._handle(SYMBOL_GROUP.get(name, "core")), name)
+        fn.restype = ctypes.c_int if name in INT_RESULT else None
+        setattr(self, name, fn)
+        return fn
+
+
+_lib = None
+
+
 def load():
-    """ctypes handle of the library; builds it when nothing is built."""
+    """Handle of the libraries (see _Libs)."""
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            build()
-        lib = ctypes.CDLL(LIB_PATH)
-        for name in ("mx_delta_rule", "mx_talk_attention",
-                     "mx_gated_delta", "mx_short_conv_silu",
-                     "mx_mfma_attention", "mx_linear_scan",
-                     "mx_linear_scan_splits",
-                     "mx_moe_route"):
-            getattr(lib, name).restype = ctypes.c_int
-        for name in ("mx_embed_scale", "mx_add_rms_norm32",
-                     "mx_add_group_norm32", "mx_group_norm_shift",
-                     "mx_depth_mix", "mx_gated_act", "mx_kv_append",
-                     "mx_attn_prep", "mx_latent_prep", "mx_norm_sum32",
-                     "mx_moe_combine",
-                     "mx_post_norm_add_norm32"):
-            getattr(lib, name).restype = None
-        _lib = lib
+        _lib = _Libs()
     return _lib
 
 
 def available() -> bool:
-    return os.path.exists(LIB_PATH)
+    return all(os.path.exists(p) for p in LIB_PATHS.values())
