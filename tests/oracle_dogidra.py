@@ -214,12 +214,15 @@ def layer(W, cfg, i, x):
     pre = f"l{i}."
     if spec["type"] != "parallel":
         raise ValueError(spec["type"])
+    conv = bool((cfg.get("canon") or {}).get("taps"))
     h = layer_norm(x, W[pre + "norm1"], W[pre + "norm1.b"], eps)
-    h = input_conv(h, W[pre + "canon1"])
+    if conv:
+        h = input_conv(h, W[pre + "canon1"])
     x = x + parallel_mixer(W, pre + "mix.", spec["mixer"], h, eps)
     if spec.get("mlp") is not None:
         h = layer_norm(x, W[pre + "norm2"], W[pre + "norm2.b"], eps)
-        h = input_conv(h, W[pre + "canon2"])
+        if conv:
+            h = input_conv(h, W[pre + "canon2"])
         x = x + routed_ff(W, pre + "mlp.", spec["mlp"], h)
     return x
 
