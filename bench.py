@@ -113,12 +113,16 @@ class User:
 # --compare-family: prefill / decode throughput of a model family beside the
 # closest existing config at equal width, depth and vocabulary (Llama for the
 # first two; for Bipulorn the other hybrid with routed feed-forwards, whose
-# expert widths are the same)
+# expert widths are the same; for Dogidra Bipulorn, whose pair layers also
+# put a windowed attention beside a recurrence ahead of a routed
+# feed-forward with a shared expert)
 COMPARE_PAIRS = {
     "nanurax": [("nanurax-1b", "llama-3.2-1b"), ("nanurax-8b", "llama-3-8b")],
     "derusun": [("derusun-1b", "llama-3.2-1b"), ("derusun-8b", "llama-3-8b")],
     "bipulorn": [("bipulorn-1b", "nanurax-1b"),
                  ("bipulorn-8b", "nanurax-8b")],
+    "dogidra": [("dogidra-1b", "bipulorn-1b"),
+                ("dogidra-8b", "bipulorn-8b")],
 }
 
 
@@ -135,6 +139,15 @@ def _truncated(name: str, layers: int) -> str:
         return name
     new = f"{name}-L{layers}"
     kw = {"name": new, "num_layers": layers}
+    if getattr(cfg, "loop", None):
+        # a looped stack is cut so that `layers` layer RUNS remain: a
+        # middle span of layers // 4 layers repeats as often as before
+        times = cfg.loop[2]
+        span = max(layers // 4, 1)
+        n = layers - (times - 1) * span
+        start = (n - span) // 2
+        kw.update(num_layers=n, loop=(start, start + span, times))
+        layers = n
     if cfg.layer_specs:
         kw["layer_specs"] = cfg.layer_specs[:layers]
     ARCHITECTURES[new] = dataclasses.replace(cfg, **kw)

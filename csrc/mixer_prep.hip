@@ -132,12 +132,13 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
   }
 }
 
-// Pooled keys/values: workgroup (segment, i) takes the i-th block of `pool`
-// positions whose last position this step appended (block b covers b*pool
-// .. b*pool + pool - 1) and stores the fp32 means of its cached keys and
-// values, rounded to the cache type, in the pooled caches [NB, G, pr, D|DV]:
-// in the page of the block's first position, at row (first position mod BS)
-// div pool.
+// Pooled keys/values: workgroup (segment, i, column chunk) takes 256
+// columns of the i-th block of `pool` positions whose last position this step
+// appended (block b covers b*pool .. b*pool + pool - 1) and stores the fp32
+// means of its cached keys and values, rounded to the cache type, in the
+// pooled caches [NB, G, pr, D|DV]: in the page of the block's first position,
+// at row (first position mod BS) div pool. A thread owns one column; its
+// loads over the block's positions are independent and run eight at a time.
 template <typename T>
 __global__ __launch_bounds__(256) void pool_append_kernel(
     const T* __restrict__ kc, const T* __restrict__ vc, T* __restrict__ kp,
@@ -148,24 +149,34 @@ __global__ __launch_bounds__(256) void pool_append_kernel(
   const int n = sr[1], p0 = sr[2];
   const int b = p0 / pool + blockIdx.y;
   if (b >= (p0 + n) / pool) return;
+  const int c = blockIdx.z * blockDim.x + threadIdx.x;
+  if (c >= G * (D + DV)) return;
   const int* table = block_tables + (size_t)blockIdx.x * max_blocks;
   const int first = b * pool;
-  const int64_t prow_base = (int64_t)table[first / BS] * G;
-  const int prow = (first % BS) / pool;
-  const float cnt = (float)pool;
-  for (int c = threadIdx.x; c < G * (D + DV); c += blockDim.x) {
-    const bool is_k = c < G * D;
-    const int cc = is_k ? c : c - G * D;
-    const int w = is_k ? D : DV;
-    const int g = cc / w, d = cc - g * w;
-    const T* cache = is_k ? kc : vc;
-    float acc = 0.f;
-    for (int j = first; j < first + pool; ++j)
-      acc += MxElem<T>::ld(
-          cache + (((int64_t)table[j / BS] * G + g) * BS + (j % BS)) * w + d);
-    T* dst = (is_k ? kp : vp) + ((prow_base + g) * pr + prow) * (int64_t)w + d;
-    MxElem<T>::st(dst, acc / cnt);
+  const bool is_k = c < G * D;
+  const int cc = is_k ? c : c - G * D;
+  const int w = is_k ? D : DV;
+  const int g = cc / w, d = cc - g * w;
+  const T* cache = (is_k ? kc : vc) + d;
+  float acc = 0.f;
+  int j = first;
+  for (; j + 8 <= first + pool; j += 8) {
+    float x[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int jj = j + u;
+      x[u] = MxElem<T>::ld(
+          cache + (((int64_t)table[jj / BS] * G + g) * BS + (jj % BS)) * w);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += x[u];
   }
+  for (; j < first + pool; ++j)
+    acc += MxElem<T>::ld(
+        cache + (((int64_t)table[j / BS] * G + g) * BS + (j % BS)) * w);
+  const int64_t prow =
+      ((int64_t)table[first / BS] * G + g) * pr + (first % BS) / pool;
+  MxElem<T>::st((is_k ? kp : vp) + prow * w + d, acc / (float)pool);
 }
 
 // Turn the pair (u, w) by the table entry (cos, sin).
@@ -324,7 +335,8 @@ void mx_pool_append(const void* kc, const void* vc, void* kp, void* vp,
   if (S_ <= 0 || blocks_per_seg <= 0 || pool < 1) return;
   const int pr = (BS + pool - 1) / pool;
   MX_DISPATCH_DTYPE(dtype, {
-    hipLaunchKernelGGL((pool_append_kernel<T>), dim3(S_, blocks_per_seg),
+    hipLaunchKernelGGL((pool_append_kernel<T>),
+                       dim3(S_, blocks_per_seg, (G * (D + DV) + 255) / 256),
                        dim3(256), 0, (hipStream_t)stream, (const T*)kc,
                        (const T*)vc, (T*)kp, (T*)vp,
                        (const int*)block_tables, max_blocks,

@@ -902,11 +902,15 @@ def mingru_scan(z: torch.Tensor, u: torch.Tensor, g: torch.Tensor,
         return out
     _check_seq_rows(seq_rows)
     assert state.is_contiguous()
+    # long segments run as tiles whose composed maps meet in this scratch
+    S = seq_rows.shape[0]
+    need = _mx().mx_mingru_scratch(S, C, T)
+    scratch = (torch.empty(need, dtype=torch.float32, device=z.device)
+               if need > 0 else None)
     _mx().mx_mingru_scan(
         _p(out), _rows(out, "out"), _p(z), _rows(z, "z"), _p(u),
         _rows(u, "u"), _p(g), _rows(g, "g"), _p(zb), _p(ub), _p(state),
-        _p(seq_rows), seq_rows.shape[0], C, T, _mx_dtype(z.dtype),
-        _stream())
+        _p(seq_rows), S, C, T, _p(scratch), _mx_dtype(z.dtype), _stream())
     return out
 
 

@@ -82,6 +82,9 @@ INT_RESULT = {
     "mx_linear_scan_splits", "mx_norm_conv32", "mx_moe_route",
 }
 
+# entry points that return a 64-bit count
+LONG_RESULT = {"mx_mingru_scratch"}
+
 
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
@@ -153,7 +156,8 @@ class _Libs:
         if not name.startswith("mx_"):
             raise AttributeError(name)
         fn = getattr(self._handle(SYMBOL_GROUP.get(name, "core")), name)
-        fn.restype = ctypes.c_int if name in INT_RESULT else None
+        fn.restype = (ctypes.c_int if name in INT_RESULT else
+                      ctypes.c_long if name in LONG_RESULT else None)
         setattr(self, name, fn)
         return fn
 
