@@ -228,6 +228,8 @@ def run_family_compare(args) -> None:
     rows = []
     for new, base in pairs:
         for name in (new, base):
+            if not name:        # "new:" measures one model alone
+                continue
             model = _truncated(name, args.compare_layers)
             r = _compare_one(model, args, use_cuda)
             rows.append(r)
@@ -244,7 +246,8 @@ def main() -> None:
                          "and decode throughput of this family beside the "
                          "closest existing config at equal size")
     ap.add_argument("--compare-models", default=None,
-                    help="new:base[,new:base] architecture names")
+                    help="new:base[,new:base] architecture names (an empty "
+                         "name is skipped)")
     ap.add_argument("--compare-layers", type=int, default=8)
     ap.add_argument("--compare-prompt-len", type=int, default=4096)
     ap.add_argument("--compare-prompts", type=int, default=4)

@@ -15,16 +15,15 @@
 #include "mix_common.h"
 
 // One wave per head: x / sqrt(mean(x^2) + eps) * w over D entries (the mean
-// over the head, or with norm_all over the whole query / key projection,
-// whose weights then have H*D / G*D entries), then the first rot_dims
-// entries turn by row `position` of the table cs [table_rows][rot_dims / 2]
-// [cos, sin]: interleaved pairs (2i, 2i+1), or with `half` pairs (i, i +
-// rot_dims / 2). A lane reads its own entries and their pair partners' and
-// only then stores, and the wave runs in step, so the query is rewritten in
-// place. Heads of up to 64 * AP_MAX_PER_LANE entries.
-#define AP_MAX_PER_LANE 8
-
-template <typename T>
+// over the head, or with ALL over the whole query / key projection, whose
+// weights then have H*D / G*D entries), then the first rot_dims entries turn
+// by row `position` of the table cs [table_rows][rot_dims / 2][cos, sin].
+// Interleaved pairs (2i, 2i+1): a lane reads its own entry and its pair
+// partner's (a neighbouring lane's) before it stores, and the wave runs in
+// step, so the query is rewritten in place. HALF pairs (i, i + rot_dims / 2):
+// a lane owns both entries of a pair, reads them, turns them and stores
+// them, so nothing it reads is another lane's to write.
+template <typename T, bool HALF, bool ALL>
 __global__ __launch_bounds__(256) void attn_prep_kernel(
     T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk,
     T* __restrict__ v, int ldv, const float* __restrict__ qw,
@@ -32,8 +31,7 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
     const T* __restrict__ vfirst, int ldvf, T* __restrict__ kc,
     T* __restrict__ vc, const int64_t* __restrict__ slots, int H, int G,
     int D, int DV, int BS, const float* __restrict__ cs, int table_rows,
-    int rot_dims, const int* __restrict__ positions, int norm_all,
-    int half) {
+    int rot_dims, const int* __restrict__ positions) {
   __shared__ float red[17];
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -47,7 +45,7 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
   // whole-projection norms: one sum of squares over all query entries and
   // one over all key entries
   float inv_q = 1.f, inv_k = 1.f;
-  if (norm_all && qw != nullptr) {
+  if (ALL && qw != nullptr) {
     float ss = 0.f;
     for (int c = threadIdx.x; c < H * D; c += blockDim.x) {
       const float x = MxElem<T>::ld(q + (size_t)t * ldq + c);
@@ -55,7 +53,7 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
     }
     inv_q = 1.0f / sqrtf(mx_block_sum(ss, red) / (float)(H * D) + eps);
   }
-  if (norm_all && kw != nullptr) {
+  if (ALL && kw != nullptr) {
     float ss = 0.f;
     for (int c = threadIdx.x; c < G * D; c += blockDim.x) {
       const float x = MxElem<T>::ld(k + (size_t)t * ldk + c);
@@ -63,18 +61,16 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
     }
     inv_k = 1.0f / sqrtf(mx_block_sum(ss, red) / (float)(G * D) + eps);
   }
-  const int hd = rot_dims >> 1;
   for (int hh = wave; hh < H + G; hh += nw) {
     const bool is_q = hh < H;
     const int g = hh - H;
     const T* src = is_q ? q + (size_t)t * ldq + hh * D
                         : k + (size_t)t * ldk + g * D;
-    const float* wgt = is_q ? qw : kw;
     // weight row of this head
-    const float* wr =
-        wgt != nullptr && norm_all ? wgt + (is_q ? hh : g) * D : wgt;
+    const float* wgt = is_q ? qw : kw;
+    if (ALL && wgt != nullptr) wgt += (is_q ? hh : g) * D;
     float inv = is_q ? inv_q : inv_k;
-    if (wgt != nullptr && !norm_all) {
+    if (!ALL && wgt != nullptr) {
       float ss = 0.f;
       for (int d = lane; d < D; d += 64) {
         const float x = MxElem<T>::ld(src + d);
@@ -89,32 +85,36 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(
     } else if (slot >= 0) {
       dst = kc + ((blk * G + g) * BS + off) * (int64_t)D;
     }
-    if (dst != nullptr) {
-      float res[AP_MAX_PER_LANE];
-#pragma unroll
-      for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
-        const int d = lane + 64 * i;
-        if (d < D) {
-          float x = MxElem<T>::ld(src + d);
-          if (wgt != nullptr) x *= inv * wr[d];
-          if (csr != nullptr && d < rot_dims) {
-            // partner entry and whether this entry is the pair's first
-            const int pd = half ? (d < hd ? d + hd : d - hd) : (d ^ 1);
-            const bool first = half ? d < hd : (d & 1) == 0;
-            const int pi = half ? (d < hd ? d : d - hd) : (d >> 1);
-            float y = MxElem<T>::ld(src + pd);
-            if (wgt != nullptr) y *= inv * wr[pd];
-            const float* e = csr + 2 * pi;
-            x = first ? x * e[0] - y * e[1] : x * e[0] + y * e[1];
-          }
-          res[i] = x;
+    if (dst == nullptr) continue;
+    if (!HALF) {
+      for (int d = lane; d < D; d += 64) {
+        float x = MxElem<T>::ld(src + d);
+        if (wgt != nullptr) x *= inv * wgt[d];
+        if (csr != nullptr && d < rot_dims) {
+          float y = MxElem<T>::ld(src + (d ^ 1));
+          if (wgt != nullptr) y *= inv * wgt[d ^ 1];
+          const float* e = csr + (d & ~1);
+          x = (d & 1) ? x * e[0] + y * e[1] : x * e[0] - y * e[1];
         }
+        MxElem<T>::st(dst + d, x);
       }
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
-        const int d = lane + 64 * i;
-        if (d < D) MxElem<T>::st(dst + d, res[i]);
+    } else {
+      const int hd = csr != nullptr ? rot_dims >> 1 : 0;
+      for (int i = lane; i < hd; i += 64) {
+        float x = MxElem<T>::ld(src + i);
+        float y = MxElem<T>::ld(src + i + hd);
+        if (wgt != nullptr) {
+          x *= inv * wgt[i];
+          y *= inv * wgt[i + hd];
+        }
+        const float c = csr[2 * i], sn = csr[2 * i + 1];
+        MxElem<T>::st(dst + i, x * c - y * sn);
+        MxElem<T>::st(dst + i + hd, y * c + x * sn);
+      }
+      for (int d = 2 * hd + lane; d < D; d += 64) {
+        float x = MxElem<T>::ld(src + d);
+        if (wgt != nullptr) x *= inv * wgt[d];
+        MxElem<T>::st(dst + d, x);
       }
     }
   }
@@ -316,15 +316,21 @@ void mx_attn_prep(void* q, int ldq, const void* k, int ldk, void* v, int ldv,
                   const void* positions, int norm_all, int half, int dtype,
                   void* stream) {
   if (T_ <= 0) return;
+#define AP_GO(HALF_, ALL_)                                                  \
+  hipLaunchKernelGGL((attn_prep_kernel<T, HALF_, ALL_>), dim3(T_), dim3(256), \
+                     0, (hipStream_t)stream, (T*)q, ldq, (const T*)k, ldk,   \
+                     (T*)v, ldv, (const float*)qw, (const float*)kw, eps,    \
+                     (const float*)vmix, (const T*)vfirst, ldvf, (T*)kc,     \
+                     (T*)vc, (const int64_t*)slots, H, G, D, DV, BS,         \
+                     (const float*)cos_sin, table_rows, rot_dims,            \
+                     (const int*)positions)
   MX_DISPATCH_DTYPE(dtype, {
-    hipLaunchKernelGGL((attn_prep_kernel<T>), dim3(T_), dim3(256), 0,
-                       (hipStream_t)stream, (T*)q, ldq, (const T*)k, ldk,
-                       (T*)v, ldv, (const float*)qw, (const float*)kw, eps,
-                       (const float*)vmix, (const T*)vfirst, ldvf, (T*)kc,
-                       (T*)vc, (const int64_t*)slots, H, G, D, DV, BS,
-                       (const float*)cos_sin, table_rows, rot_dims,
-                       (const int*)positions, norm_all, half);
+    if (half && norm_all) AP_GO(true, true);
+    else if (half) AP_GO(true, false);
+    else if (norm_all) AP_GO(false, true);
+    else AP_GO(false, false);
   })
+#undef AP_GO
 }
 
 void mx_pool_append(const void* kc, const void* vc, void* kp, void* vp,
