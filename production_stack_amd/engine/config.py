@@ -711,8 +711,8 @@ def _dogidra_stack(
     attn_kv: int, attn_dim: int, attn_vdim: int, window: int, pool: int,
     rot_dims: int, rot_scaling: Optional[tuple], gru: int, experts: int,
     top: int, expert_ff: int, shared_ff: int, taps: int, loop: tuple,
-    softcap: float = 30.0, route_scale: float = 2.5,
-    left_scale: float = 0.8, right_scale: float = 0.5,
+    softcap: float = 50.0, route_scale: float = 2.0,
+    left_scale: float = 1.0, right_scale: float = 1.0,
     embedding_scale: float = 1.0,
 ) -> ModelConfig:
     """A Dogidra stack: every layer a pair of windowed attention with
@@ -726,7 +726,7 @@ def _dogidra_stack(
             kind="attention", heads=attn_heads, kv_heads=attn_kv,
             dim=attn_dim, vdim=attn_vdim, scale=attn_dim ** -0.5,
             window=window, window_pool=pool, softcap=softcap, rope=True,
-            rot_dims=rot_dims, rot_base=50000.0, rot_layout="half",
+            rot_dims=rot_dims, rot_base=10000.0, rot_layout="half",
             rot_scaling=rot_scaling, qk_norm_all=True)
         right = MixerSpec(kind="mingru", heads=1, dim=1, vdim=gru,
                           rope=False)
@@ -755,7 +755,7 @@ ARCHITECTURES.update({
     "tiny-dogidra": _dogidra_stack(
         "tiny-dogidra", 96, 384, 4, attn_heads=6, attn_kv=3, attn_dim=16,
         attn_vdim=8, window=40, pool=8, rot_dims=8,
-        rot_scaling=(4.0, 64, 8.0, 1.0), gru=128, experts=5, top=2,
+        rot_scaling=(2.0, 64, 8.0, 1.0), gru=128, experts=5, top=2,
         expert_ff=32, shared_ff=64, taps=3, loop=(1, 3, 2),
         embedding_scale=8.0),
     # llama-3.2-1b-sized stack (same width and vocab; 12 layers, the middle
@@ -763,13 +763,13 @@ ARCHITECTURES.update({
     "dogidra-1b": _dogidra_stack(
         "dogidra-1b", 2048, 128256, 12, attn_heads=32, attn_kv=8,
         attn_dim=64, attn_vdim=64, window=1024, pool=64, rot_dims=64,
-        rot_scaling=(4.0, 2048, 32.0, 1.0), gru=4096, experts=8, top=2,
+        rot_scaling=(8.0, 2048, 16.0, 1.0), gru=4096, experts=8, top=2,
         expert_ff=2048, shared_ff=2048, taps=4, loop=(4, 8, 2)),
     # llama-3-8b-sized layers (width 4096, head dim 128)
     "dogidra-8b": _dogidra_stack(
         "dogidra-8b", 4096, 128256, 24, attn_heads=32, attn_kv=8,
         attn_dim=128, attn_vdim=128, window=2048, pool=64, rot_dims=128,
-        rot_scaling=(4.0, 2048, 32.0, 1.0), gru=8192, experts=8, top=2,
+        rot_scaling=(8.0, 2048, 16.0, 1.0), gru=8192, experts=8, top=2,
         expert_ff=3584, shared_ff=3584, taps=4, loop=(8, 16, 2)),
 })
 

@@ -32,7 +32,7 @@ def close(got, want, dtype):
 
 def mixer(heads=4, kv_heads=2, dim=16, vdim=24, size=20, pool=4, scale=0.3,
           rot_dims=8, base=100.0, scaling=(4.0, 32, 4.0, 1.0), softcap=15.0,
-          gru=40, left_scale=0.8, right_scale=0.5):
+          gru=40, left_scale=0.7, right_scale=0.6):
     left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
             "scale": scale}
     if softcap:

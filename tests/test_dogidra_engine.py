@@ -30,8 +30,8 @@ STACK = [
     (mixer(4, 2, 16, 24, 20, 4, 0.3, 8, 100.0, (4.0, 32, 4.0, 1.0), 15.0, 40),
      moe(24, 5, 2, 1.5, 40)),
     (mixer(6, 3, 8, 8, 13, 5, 0.4, 8, 10000.0, None, 0.0, 24, 1.0, 1.0),
-     moe(16, 4, 3, 2.5, 0)),
-    (mixer(2, 1, 16, 8, 20, 4, 0.25, 4, 50.0, (2.0, 16, 2.0, 0.5), 30.0, 40,
+     moe(16, 4, 3, 2.25, 0)),
+    (mixer(2, 1, 16, 8, 20, 4, 0.25, 4, 50.0, (2.0, 16, 2.0, 0.5), 22.0, 40,
            0.5, 1.5), None),
     (mixer(4, 4, 16, 16, 33, 16, 0.3, 16, 1000.0, (8.0, 64, 8.0, 1.0), 10.0,
            8), moe(24, 3, 1, 1.0, 24)),
@@ -83,7 +83,7 @@ def test_registry_reads_checkpoint_folder(ckpt):
     assert s0.norm == "layer" and s0.input_conv == 3 and not s0.parallel
     m0 = s0.mixer
     assert (m0.kind, m0.combine, m0.left_scale, m0.right_scale) == (
-        "pair", "weighted", 0.8, 0.5)
+        "pair", "weighted", 0.7, 0.6)
     a, b = m0.left, m0.right
     assert (a.kind, a.heads, a.kv_heads, a.dim, a.vdim, a.window,
             a.window_pool, a.scale, a.softcap, a.rot_dims, a.rot_base,
@@ -98,6 +98,7 @@ def test_registry_reads_checkpoint_folder(ckpt):
         5, 2, 1.5, 40, True, "sigmoid", "relu2", False, False, False)
     assert s1.mixer.left.rot_scaling is None and s1.mixer.left.softcap == 0
     assert s1.mlp.shared_ff == 0 and s2.mlp is None
+    assert s1.mlp.route_scale == 2.25
     assert "dogidra" in registry.FP32_FAMILIES
     model = registry.build_model(mc, "float32")
     assert [i for i, _ in model.runs] == [0, 1, 2, 1, 2, 3]
@@ -264,11 +265,11 @@ OTHER_STACKS = [
      60, 71, 1e-5, 7, (2, 3, 1), 3.0),
     # only the last layer looped, twice; an empty looped span elsewhere is
     # not needed: start == stop gives passes without layers
-    ([(mixer(2, 2, 32, 32, 16, 16, 0.18, 32, 5e4, (4.0, 64, 32.0, 1.0), 30.0,
-             48), moe(24, 4, 2, 2.5, 24)),
-      (mixer(8, 1, 16, 8, 24, 8, 0.25, 16, 5e4, (4.0, 64, 32.0, 1.0), 30.0,
+    ([(mixer(2, 2, 32, 32, 16, 16, 0.18, 32, 2e4, (3.0, 48, 16.0, 1.0), 25.0,
+             48), moe(24, 4, 2, 1.75, 24)),
+      (mixer(8, 2, 16, 8, 24, 8, 0.25, 16, 2e4, (3.0, 48, 16.0, 1.0), 25.0,
              40), moe(8, 7, 3, 1.0, 0))],
-     64, 37, 1e-5, 4, (1, 2, 2), 12.0),
+     64, 37, 1e-5, 5, (1, 2, 2), 7.0),
 ]
 
 
