@@ -875,7 +875,7 @@ def add_layer_norm_conv32(x32: torch.Tensor, deltas, scales,
             _stream())
         if rc != 0:
             raise RuntimeError(
-                f"add_layer_norm_conv32: {K} taps are not built (1-8)")
+                f"add_layer_norm_conv32: {K} taps are not built (1-32)")
     return h
 
 

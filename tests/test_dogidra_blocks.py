@@ -277,10 +277,12 @@ def gtol(dtype):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("K", [0, 1, 2, 4, 8])
-def test_gpu_layer_norm_conv(dtype, K):
+@pytest.mark.parametrize("K", [0, 1, 2, 4, 8, 11])
+@pytest.mark.parametrize("W_", [328, 330])
+def test_gpu_layer_norm_conv(dtype, K, W_):
+    """Row widths with and without whole 16-byte vectors; tap counts with
+    their own instantiation (up to 8) and above."""
     g = torch.Generator().manual_seed(10 + K)
-    W_ = 328
     lens, pos0, slots = [70, 1, 3, 130, 1], [0, 5, 2, 64, 0], [3, 0, 2, 1, 4]
     sr, T = segments(lens, pos0, slots)
     x = rnd(g, T, W_, scale=2.0) + 0.5
