@@ -25,11 +25,18 @@
 
 #define MG_TILE 128
 
+// Three sigmoids per element make these kernels arithmetic-bound with the
+// library's range-checked exponential and IEEE division, so they use the
+// hardware exponential and reciprocal (fp32, a few ulp).
+PS_DEV float mg_sigmoid(float x) {
+  return __fdividef(1.0f, 1.0f + __expf(-x));
+}
+
 PS_DEV void mg_gate(float zv, float uv, float bz, float bu, float* a,
                     float* cand) {
-  *a = mx_sigmoid(zv + bz);
+  *a = mg_sigmoid(zv + bz);
   const float uu = uv + bu;
-  *cand = uu >= 0.f ? uu + 0.5f : mx_sigmoid(uu);
+  *cand = uu >= 0.f ? uu + 0.5f : mg_sigmoid(uu);
 }
 
 template <typename T>
@@ -52,7 +59,7 @@ __global__ __launch_bounds__(64) void mingru_scan_kernel(
             bz, bu, &a, &cand);
     const float gg = MxElem<T>::ld(g + t * ldg + c);
     S = (1.0f - a) * S + a * cand;
-    MxElem<T>::st(out + t * ldo + c, S * (gg * mx_sigmoid(gg)));
+    MxElem<T>::st(out + t * ldo + c, S * (gg * mg_sigmoid(gg)));
   }
   state[(size_t)slot * C + c] = S;
 }
@@ -118,7 +125,7 @@ __global__ __launch_bounds__(64) void mingru_tile_scan_kernel(
             bz, bu, &a, &cand);
     const float gg = MxElem<T>::ld(g + t * ldg + c);
     S = (1.0f - a) * S + a * cand;
-    MxElem<T>::st(out + t * ldo + c, S * (gg * mx_sigmoid(gg)));
+    MxElem<T>::st(out + t * ldo + c, S * (gg * mg_sigmoid(gg)));
   }
   if (r1 == n) state[(size_t)slot * C + c] = S;
 }

@@ -309,20 +309,23 @@ def test_gpu_layer_norm_conv(dtype, K, W_):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_gpu_mingru_scan(dtype):
+@pytest.mark.parametrize("pad", [5, 0])
+def test_gpu_mingru_scan(dtype, pad):
+    """Ragged segments above and below the tile length; row strides and
+    offsets with (pad 0) and without whole 16-byte vectors."""
     g = torch.Generator().manual_seed(11)
     C = 200
     lens, pos0, slots = [90, 1, 2, 300, 1], [0, 7, 0, 16, 3], [2, 4, 0, 1, 3]
     sr, T = segments(lens, pos0, slots)
-    big = rnd(g, T, 3 * C + 5).to(dtype)
-    z, u, gate = big[:, :C], big[:, C:2 * C], big[:, 2 * C + 5:]
+    big = rnd(g, T, 3 * C + pad).to(dtype)
+    z, u, gate = big[:, :C], big[:, C:2 * C], big[:, 2 * C + pad:]
     zb, ub = rnd(g, C), rnd(g, C)
     st = rnd(g, 5, C)
     st_ref = st.clone()
     want = R.mingru_scan(z, u, gate, zb, ub, st_ref, sr, dtype)
     st_gpu = st.cuda()
     bg = big.cuda()
-    got = ops.mingru_scan(bg[:, :C], bg[:, C:2 * C], bg[:, 2 * C + 5:],
+    got = ops.mingru_scan(bg[:, :C], bg[:, C:2 * C], bg[:, 2 * C + pad:],
                           zb.cuda(), ub.cuda(), st_gpu, sr.cuda())
     assert relerr(got, want) < gtol(dtype)
     assert relerr(st_gpu, st_ref) < 1e-5
