@@ -116,7 +116,9 @@ PS_DEV void mf_stage(unsigned short* __restrict__ dst, int pitch,
   }
 }
 
-template <int CBW, int ROWS>
+// POOL: the instantiation with the pooled range; without it the kernel is
+// the two-range form the families without pooled blocks have always run.
+template <int CBW, int ROWS, bool POOL>
 __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
     unsigned short* __restrict__ out, int ldout,
     const unsigned short* __restrict__ q, int ldq,
@@ -183,7 +185,7 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
   const bool valid = my_i < ntok;  // ntok <= TPB
   const int my_pos = valid ? s_pos[my_i] : 0;
   const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
-  const int my_pool = opt.kp ? mf_pool_count(my_pos, window, opt.pool) : 0;
+  const int my_pool = POOL ? mf_pool_count(my_pos, window, opt.pool) : 0;
   const float inv_cap2 = opt.softcap > 0.f ? 2.0f / opt.softcap : 0.f;
   const bool own_sink = sink && ks == 0;
   float m = own_sink ? (opt.sink_vals ? opt.sink_vals[my_head] : 0.f)
@@ -209,12 +211,13 @@ __global__ __launch_bounds__(256, 2) void mfma_attn_kernel(
     // kept first keys behind the run's earliest window, the pooled blocks
     // its last row sees, then the windows
     const int run_pool =
-        opt.kp ? mf_pool_count(s_pos[re - 1], window, opt.pool) : 0;
-    for (int rg = 0; rg < 3; ++rg) {
-      const int ra = rg == 2 ? kmin : 0;
+        POOL ? mf_pool_count(s_pos[re - 1], window, opt.pool) : 0;
+    constexpr int NR = POOL ? 3 : 2;
+    for (int rg = 0; rg < NR; ++rg) {
+      const bool pl = POOL && rg == 1;
+      const int ra = rg == NR - 1 ? kmin : 0;
       const int rb = rg == 0 ? min(opt.keep_first, kmin) - 1
-                             : (rg == 1 ? run_pool - 1 : kmax);
-      const bool pl = rg == 1;
+                             : (pl ? run_pool - 1 : kmax);
       for (int j0 = ra; j0 <= rb; j0 += 32, ++tile_no) {
         if (tile_no % KS != ks) continue;
         const int nk = min(32, rb + 1 - j0);
@@ -405,8 +408,8 @@ static size_t mf_lds_budget(const void* fn) {
   return 64 * 1024;
 }
 
-template <int CBW, int ROWS>
-static int mf_launch(void* out, int ldout, const void* q, int ldq,
+template <int CBW, int ROWS, bool POOL>
+static int mf_launch_as(void* out, int ldout, const void* q, int ldq,
                      const void* kc, const void* vc, const void* block_tables,
                      int max_blocks, const void* token_seq,
                      const void* token_pos, int T_, int H, int G, int D,
@@ -414,7 +417,7 @@ static int mf_launch(void* out, int ldout, const void* q, int ldq,
                      MfOpt opt, int KS, float* part, int tpb_max,
                      hipStream_t stream) {
   static const size_t budget =
-      mf_lds_budget((const void*)mfma_attn_kernel<CBW, ROWS>);
+      mf_lds_budget((const void*)mfma_attn_kernel<CBW, ROWS, POOL>);
   const int DP = (D + 15) & ~15, PK = DP + 8;
   const int DVP = (DV + 31) & ~31;
   const size_t lds = ((size_t)(ROWS + 32) * PK +
@@ -424,7 +427,7 @@ static int mf_launch(void* out, int ldout, const void* q, int ldq,
   const int HPB = rep < 32 ? rep : 32;
   const int TPB = ROWS / HPB < tpb_max ? ROWS / HPB : tpb_max;
   dim3 grid((T_ + TPB - 1) / TPB, G * (rep / HPB), KS);
-  hipLaunchKernelGGL((mfma_attn_kernel<CBW, ROWS>), grid, dim3(256), lds,
+  hipLaunchKernelGGL((mfma_attn_kernel<CBW, ROWS, POOL>), grid, dim3(256), lds,
                      stream,
                      (unsigned short*)out, ldout, (const unsigned short*)q,
                      ldq, (const unsigned short*)kc,
@@ -438,6 +441,25 @@ static int mf_launch(void* out, int ldout, const void* q, int ldq,
                        stream, (unsigned short*)out, ldout,
                        (const float*)part, H, DV, KS);
   return 0;
+}
+
+template <int CBW, int ROWS>
+static int mf_launch(void* out, int ldout, const void* q, int ldq,
+                     const void* kc, const void* vc, const void* block_tables,
+                     int max_blocks, const void* token_seq,
+                     const void* token_pos, int T_, int H, int G, int D,
+                     int DV, int BS, float scale, int window, int sink,
+                     MfOpt opt, int KS, float* part, int tpb_max,
+                     hipStream_t stream) {
+  if (opt.kp != nullptr)
+    return mf_launch_as<CBW, ROWS, true>(
+        out, ldout, q, ldq, kc, vc, block_tables, max_blocks, token_seq,
+        token_pos, T_, H, G, D, DV, BS, scale, window, sink, opt, KS, part,
+        tpb_max, stream);
+  return mf_launch_as<CBW, ROWS, false>(
+      out, ldout, q, ldq, kc, vc, block_tables, max_blocks, token_seq,
+      token_pos, T_, H, G, D, DV, BS, scale, window, sink, opt, KS, part,
+      tpb_max, stream);
 }
 
 // Returns 0 when launched, 1 when the shape is outside this kernel (the

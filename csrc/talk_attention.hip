@@ -50,6 +50,7 @@ PS_DEV int ta_pool_count(int pos, int window, int pool) {
 // P positions (the key/value cache: P = 1, R = BS).
 PS_DEV int64_t ta_row(const int* __restrict__ table, int j, int G, int g,
                       int BS, int P, int R) {
+  if (P == 1) return ((int64_t)table[j / BS] * G + g) * BS + (j % BS);
   const int pos = j * P;
   return ((int64_t)table[pos / BS] * G + g) * R + (pos % BS) / P;
 }
