@@ -162,7 +162,9 @@ def test_long_decode_past_many_windows_and_blocks(ckpt, device):
     toks = tokens(260, 3)
     want = O.forward(cfg, W, toks)
     eng = make_engine(path, "float32", device)
-    got = replay(eng, "a", toks, [37] + [1] * 223)
+    # a first portion of more than 128 rows routes through the sorted
+    # expert dispatch, the single tokens through the all-experts path
+    got = replay(eng, "a", toks, [137] + [1] * 123)
     assert rel_err(got, want) < TOL["float32"]
 
 
