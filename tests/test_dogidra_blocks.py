@@ -42,13 +42,15 @@ def relerr(a, b):
 class PagedAttention:
     def __init__(self, m, Wq, Wk, Wv, qn, kn, eps, bs=8, pages=None,
                  device="cpu", dtype=torch.float32, n_pages=64, seed=0):
-        self.m, self.eps, self.bs, self.dev, self.dt = m, eps, bs, device, dtype
+        self.m, self.eps, self.bs = m, eps, bs
+        self.dev, self.dt = device, dtype
         self.H, self.G = m["heads"], m.get("kv_heads", m["heads"])
         self.D, self.DV = m["dim"], m.get("vdim", m["dim"])
         self.W = [w.to(dtype).to(device) for w in (Wq, Wk, Wv)]
         self.qn, self.kn = qn.float().to(device), kn.float().to(device)
         mask = m.get("mask") or {}
-        self.window, self.P = int(mask.get("size", 0)), int(mask.get("pool", 0))
+        self.window = int(mask.get("size", 0))
+        self.P = int(mask.get("pool", 0))
         rot = m.get("rot") or {}
         self.rot_dims = int(rot.get("dims", 0))
         sc = rot.get("scaling")
@@ -60,8 +62,10 @@ class PagedAttention:
                 if sc else None)
         g = torch.Generator().manual_seed(seed)
         # caches start full of another owner's numbers
-        mk = lambda r, w: (torch.randn(n_pages, self.G, r, w, generator=g)  # noqa: E731,E501
-                           * 3).to(dtype).to(device)
+        def mk(r, w):
+            return (torch.randn(n_pages, self.G, r, w, generator=g)
+                    * 3).to(dtype).to(device)
+
         self.kc, self.vc = mk(bs, self.D), mk(bs, self.DV)
         self.pool = None
         if self.P:
@@ -126,7 +130,7 @@ def oracle_attention(m, W, h, eps):
 
 @pytest.mark.parametrize("case", [
     dict(),                                        # everything on
-    dict(pool=1),                                  # every far token its own block
+    dict(pool=1),                                  # blocks of one position
     dict(pool=16, size=5),                         # blocks longer than a page
     dict(pool=0),                                  # window only
     dict(size=0, pool=0),                          # plain causal
